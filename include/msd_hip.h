@@ -1,0 +1,128 @@
+/*
+ * msd_hip.h - C ABI of the MI355X (gfx950) norm / activation / embedding kernels.
+ *
+ * Plain C: pointers, sizes, ints.  Every device pointer is HIP device memory on
+ * the current device; `stream` is a hipStream_t passed as void* (NULL = the
+ * default stream).  Calls are asynchronous on that stream.  Return value: 0 on
+ * success, otherwise a hipError_t value (1 = hipErrorInvalidValue is also used
+ * for rejected shapes / null pointers / unknown dtype).  No call throws.
+ *
+ * Each entry point names the reference interface it replaces (paths relative to
+ * app/src/main of 9Hyeonwoo/mobile-stable-diffusion; K/ = assets/kernel/,
+ * M/ = cpp/modules/).  The reference is fp32, batch 1; `dtype` and `batch` are
+ * extensions.  gamma / beta are always float32.
+ */
+#ifndef MSD_HIP_H
+#define MSD_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MSD_OK 0
+#define MSD_ERR_INVALID_VALUE 1 /* == hipErrorInvalidValue */
+
+/* storage type of activations; arithmetic is always float32 */
+#define MSD_DTYPE_F32 0
+#define MSD_DTYPE_F16 1
+
+/* Library version: major*10000 + minor*100 + patch. */
+int msd_version(void);
+
+/* Human-readable text for a return code (static storage). */
+const char *msd_error_string(int code);
+
+/*
+ * Creates the per-(device, stream) scratch (a few MiB, holds the partial
+ * statistics that workgroups sharing one GroupNorm group exchange) ahead of
+ * time.  Optional: msd_groupnorm creates it on first use; call this first
+ * when the first msd_groupnorm on a stream would otherwise happen under
+ * stream capture.  No reference counterpart (the reference allocates two
+ * temporaries per forward, M/nn/GroupNorm.cpp:95-103).
+ */
+int msd_init(void *stream);
+
+/* Frees every scratch buffer created so far on all devices. */
+int msd_shutdown(void);
+
+/*
+ * Synchronises `stream` and reports whether any msd_groupnorm launched on it
+ * so far gave up waiting for a sibling workgroup (its output is then invalid):
+ * 0, or hipErrorLaunchFailure.  The flag is sticky.  No reference counterpart.
+ */
+int msd_status(void *stream);
+
+/*
+ * Tuning knob: msd_groupnorm splits each (sample, group) over enough
+ * workgroups to reach about this many per launch (default 512).
+ */
+int msd_set_groupnorm_target_blocks(int blocks);
+
+/*
+ * GroupNorm over NCHW, optionally followed by SiLU, in one launch.
+ * Replaces the 3-kernel chain enqueued by GroupNorm::forward
+ * (M/nn/GroupNorm.cpp:105-145; K/group_norm.cl:1-76) and, with fuse_silu != 0,
+ * the separate silu enqueue that follows it (M/nn/ResBlock.cpp:136-142,
+ * K/util.cl:124-134).  Biased variance, y = fma((x-mean)/sqrt(var+eps), gamma[c],
+ * beta[c]).  x and y are [batch, channels, hw]; y may alias x exactly (in place,
+ * M/nn/ResBlock.cpp:222).  Requires channels % groups == 0.
+ */
+int msd_groupnorm(const void *x, void *y, const float *gamma, const float *beta,
+                  size_t batch, size_t channels, size_t hw, size_t groups, float eps,
+                  int fuse_silu, int dtype, void *stream);
+
+/*
+ * LayerNorm over the last dimension of a row-major [rows, dim] tensor.
+ * Replaces LayerNorm::forward (M/nn/LayerNorm.cpp:94-139; K/layer_norm.cl:1-78);
+ * the reference's eps is the constant 1e-5 (K/layer_norm.cl:58).  y may alias x.
+ */
+int msd_layernorm(const void *x, void *y, const float *gamma, const float *beta, size_t rows,
+                  size_t dim, float eps, int dtype, void *stream);
+
+/*
+ * GEGLU epilogue on an already projected tensor: proj is [rows, 2*inner] with
+ * the value in the first half of each row and the gate in the second;
+ * out[r, c] = proj[r, c] * gelu_erf(proj[r, inner + c]).  Replaces the
+ * gelu_multiply enqueue of GEGLU::forward (M/nn/GEGLU.cpp:71-78; K/geglu.cl:1-25).
+ * out must not overlap proj.
+ */
+int msd_geglu(const void *proj, void *out, size_t rows, size_t inner, int dtype, void *stream);
+
+/*
+ * Elementwise activations over n elements; y may alias x (every reference call
+ * site is in place).
+ *   msd_silu       K/util.cl:124-134 (enqueued at M/nn/ResBlock.cpp:136-142,173-180,
+ *                  225-232; M/UNetModel.cpp:1110-1117,1803-1810)
+ *   msd_gelu       K/util.cl:104-122 (M/nn/ResidualAttentionBlock.cpp:146-153), erf form
+ *   msd_quick_gelu x*sigmoid(1.702x); no reference counterpart
+ */
+int msd_silu(const void *x, void *y, size_t n, int dtype, void *stream);
+int msd_gelu(const void *x, void *y, size_t n, int dtype, void *stream);
+int msd_quick_gelu(const void *x, void *y, size_t n, int dtype, void *stream);
+
+/*
+ * Sinusoidal timestep embedding, out[b] = [cos(t_b*f_i) | sin(t_b*f_i)],
+ * f_i = exp(-log(max_period) * i / (dim/2)), i < dim/2.  Replaces the host loop
+ * UNetModel::createTimestepEmbedding (M/UNetModel.cpp:1935-1958): same float32
+ * expression for f_i and t*f_i.  timesteps is a device array of `batch` int64
+ * values, out is [batch, dim]; dim must be even.
+ */
+int msd_timestep_embedding(const int64_t *timesteps, void *out, size_t batch, size_t dim,
+                           float max_period, int dtype, void *stream);
+
+/*
+ * Integer DDIM timestep list (host only, no GPU work): c = 1000 / steps;
+ * {1, 1+c, 1+2c, ...} while < 1000+1, ascending, exactly as
+ * DDIMSampler::sample builds it (M/DDIMSampler.cpp:60-64); the sampler walks it
+ * from the back (M/DDIMSampler.cpp:78-82).  Writes at most cap entries and
+ * returns the full count, or -1 for steps outside [1, 1000].
+ */
+int msd_ddim_timesteps(int ddim_num_steps, int *out, int cap);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MSD_HIP_H */

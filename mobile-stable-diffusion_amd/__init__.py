@@ -1,0 +1,171 @@
+"""ctypes access to the MI355X norm / activation / embedding library.
+
+The product is the native code under csrc/ (HIP kernels behind the C ABI of
+include/msd_hip.h, and the C++ layer objects on top of it).  This module only
+loads the built libraries and passes torch tensors' device pointers and the
+current torch stream through the C ABI; torch is used for device memory and
+streams, nothing else.  There is no fallback: if the library was not built
+the loader raises.
+"""
+import ctypes
+import os
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+CSRC_DIR = os.path.join(_PKG_DIR, "csrc")
+LIB_HIP_PATH = os.path.join(CSRC_DIR, "libmsd_hip.so")
+LIB_NN_PATH = os.path.join(CSRC_DIR, "libmsd_nn.so")
+
+DTYPE_F32 = 0
+DTYPE_F16 = 1
+
+# every symbol include/msd_hip.h declares
+C_ABI_SYMBOLS = (
+    "msd_version", "msd_error_string", "msd_init", "msd_shutdown", "msd_status",
+    "msd_set_groupnorm_target_blocks", "msd_groupnorm", "msd_layernorm", "msd_geglu",
+    "msd_silu", "msd_gelu", "msd_quick_gelu", "msd_timestep_embedding", "msd_ddim_timesteps",
+)
+
+_lib = None
+
+
+class MsdError(RuntimeError):
+    pass
+
+
+def load_library(path=None):
+    """Loads libmsd_hip.so (built in-tree) and declares the C ABI signatures."""
+    global _lib
+    if _lib is not None and path is None:
+        return _lib
+    path = path or LIB_HIP_PATH
+    if not os.path.exists(path):
+        raise MsdError(
+            "native library %s is missing: build it with `python -c 'import __graft_entry__ as g;"
+            " g.build()'` (there is no non-native fallback)" % path)
+    lib = ctypes.CDLL(path, mode=ctypes.RTLD_GLOBAL)
+    vp, sz, fl, it = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float, ctypes.c_int
+    lib.msd_version.restype = it
+    lib.msd_error_string.restype = ctypes.c_char_p
+    lib.msd_error_string.argtypes = [it]
+    lib.msd_init.argtypes = [vp]
+    lib.msd_shutdown.argtypes = []
+    lib.msd_status.argtypes = [vp]
+    lib.msd_set_groupnorm_target_blocks.argtypes = [it]
+    lib.msd_groupnorm.argtypes = [vp, vp, vp, vp, sz, sz, sz, sz, fl, it, it, vp]
+    lib.msd_layernorm.argtypes = [vp, vp, vp, vp, sz, sz, fl, it, vp]
+    lib.msd_geglu.argtypes = [vp, vp, sz, sz, it, vp]
+    for name in ("msd_silu", "msd_gelu", "msd_quick_gelu"):
+        getattr(lib, name).argtypes = [vp, vp, sz, it, vp]
+    lib.msd_timestep_embedding.argtypes = [vp, vp, sz, sz, fl, it, vp]
+    lib.msd_ddim_timesteps.argtypes = [it, ctypes.POINTER(ctypes.c_int), it]
+    for name in C_ABI_SYMBOLS:
+        if name != "msd_error_string":
+            getattr(lib, name).restype = it
+    _lib = lib
+    return lib
+
+
+def check(code):
+    if code != 0:
+        raise MsdError("msd call failed with code %d: %s"
+                       % (code, load_library().msd_error_string(code).decode()))
+
+
+def _dtype_code(t):
+    import torch
+    if t.dtype == torch.float32:
+        return DTYPE_F32
+    if t.dtype == torch.float16:
+        return DTYPE_F16
+    raise MsdError("unsupported storage dtype %s" % t.dtype)
+
+
+def _stream():
+    import torch
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dev(t):
+    if not t.is_cuda or not t.is_contiguous():
+        raise MsdError("expected a contiguous device tensor")
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def init():
+    check(load_library().msd_init(_stream()))
+
+
+def status():
+    return load_library().msd_status(_stream())
+
+
+def groupnorm(x, gamma, beta, groups, eps=1e-5, fuse_silu=False, out=None):
+    """x: [batch, C, ...] device tensor; gamma/beta float32 [C]; out may be x (in place)."""
+    import torch
+    out = torch.empty_like(x) if out is None else out
+    batch, channels = x.shape[0], x.shape[1]
+    hw = x.numel() // (batch * channels) if batch * channels else 0
+    check(load_library().msd_groupnorm(_dev(x), _dev(out), _dev(gamma), _dev(beta), batch, channels,
+                                       hw, groups, eps, int(fuse_silu), _dtype_code(x), _stream()))
+    return out
+
+
+def layernorm(x, gamma, beta, eps=1e-5, out=None):
+    import torch
+    out = torch.empty_like(x) if out is None else out
+    dim = x.shape[-1]
+    rows = x.numel() // dim if dim else 0
+    check(load_library().msd_layernorm(_dev(x), _dev(out), _dev(gamma), _dev(beta), rows, dim, eps,
+                                       _dtype_code(x), _stream()))
+    return out
+
+
+def geglu(proj, out=None):
+    """proj: [..., 2*inner] (value | gate) -> [..., inner]."""
+    import torch
+    inner = proj.shape[-1] // 2
+    rows = proj.numel() // (2 * inner) if inner else 0
+    if out is None:
+        out = torch.empty(proj.shape[:-1] + (inner,), dtype=proj.dtype, device=proj.device)
+    check(load_library().msd_geglu(_dev(proj), _dev(out), rows, inner, _dtype_code(proj), _stream()))
+    return out
+
+
+def _act(name, x, out):
+    import torch
+    out = torch.empty_like(x) if out is None else out
+    check(getattr(load_library(), name)(_dev(x), _dev(out), x.numel(), _dtype_code(x), _stream()))
+    return out
+
+
+def silu(x, out=None):
+    return _act("msd_silu", x, out)
+
+
+def gelu(x, out=None):
+    return _act("msd_gelu", x, out)
+
+
+def quick_gelu(x, out=None):
+    return _act("msd_quick_gelu", x, out)
+
+
+def timestep_embedding(timesteps, dim, max_period=10000.0, dtype=None):
+    """timesteps: int64 device tensor [batch] -> [batch, dim] as [cos | sin]."""
+    import torch
+    dtype = dtype or torch.float32
+    out = torch.empty((timesteps.numel(), dim), dtype=dtype, device=timesteps.device)
+    check(load_library().msd_timestep_embedding(_dev(timesteps), _dev(out), timesteps.numel(), dim,
+                                                max_period, _dtype_code(out), _stream()))
+    return out
+
+
+def ddim_timesteps(steps):
+    """Ascending integer DDIM timestep list (host only)."""
+    lib = load_library()
+    n = lib.msd_ddim_timesteps(steps, None, 0)
+    if n < 0:
+        raise MsdError("ddim steps must be in [1, 1000]")
+    buf = (ctypes.c_int * n)()
+    lib.msd_ddim_timesteps(steps, buf, n)
+    return list(buf)

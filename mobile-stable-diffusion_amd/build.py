@@ -1,0 +1,73 @@
+"""Build recipe for the native libraries (hipcc cross-compiles gfx950 without a GPU).
+
+    libmsd_hip.so   HIP kernels + the C ABI declared in include/msd_hip.h
+    libmsd_nn.so    C++ host layer objects (GroupNorm / LayerNorm / GEGLU / ...) on top of it
+
+Run as a script (`python build.py`) or call build_all().
+"""
+import os
+import subprocess
+import sys
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(PKG_DIR, "csrc")
+REPO = os.path.dirname(PKG_DIR)
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+ARCH = "gfx950"
+# -packed-fp32-ops is switched off: plain float code must not be turned into
+# v_pk_*_f32 instructions.
+DEVICE_FLAGS = [
+    "-O3", "-std=c++17", f"--offload-arch={ARCH}", "-fPIC",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+LIB_HIP = os.path.join(CSRC, "libmsd_hip.so")
+LIB_NN = os.path.join(CSRC, "libmsd_nn.so")
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines()
+                    if "is not a recognized feature for this target" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError("build failed: %s\n%s" % (" ".join(cmd), out))
+    return out
+
+
+def build_hip():
+    src = os.path.join(CSRC, "msd_kernels.hip")
+    _run([HIPCC] + DEVICE_FLAGS + ["-shared", "-o", LIB_HIP, src])
+    return LIB_HIP
+
+
+def build_nn():
+    nn_dir = os.path.join(CSRC, "nn")
+    srcs = sorted(os.path.join(nn_dir, f) for f in os.listdir(nn_dir) if f.endswith(".cpp"))
+    if not srcs:
+        return None
+    # host-only C++; hipcc is used for the HIP runtime include / link paths
+    cmd = [HIPCC, "-O2", "-std=c++17", "-fPIC", "-shared", "-x", "c++",
+           "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(REPO, "include"), "-I", nn_dir,
+           "-Wall", "-Wno-unused-command-line-argument"] + srcs + [
+           "-o", LIB_NN, "-L", CSRC, "-lmsd_hip", "-Wl,-rpath,$ORIGIN", "-lamdhip64",
+           "-L/opt/rocm/lib"]
+    _run(cmd)
+    return LIB_NN
+
+
+def build_all(verbose=True):
+    built = [build_hip()]
+    nn = build_nn()
+    if nn:
+        built.append(nn)
+    if verbose:
+        for b in built:
+            print("built", b)
+    return built
+
+
+if __name__ == "__main__":
+    build_all()
+    sys.exit(0)

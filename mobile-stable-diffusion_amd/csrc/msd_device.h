@@ -1,0 +1,191 @@
+// Device-side building blocks shared by the gfx950 kernels: 16-byte packed
+// access for float / half storage, DPP reductions for 64-wide wavefronts,
+// activation math, and a multiply-shift replacement for integer division.
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace msd {
+
+constexpr int kWave = 64;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// ---------------------------------------------------------------------------
+// Storage traits: one 16-byte vector holds EPV elements.
+// ---------------------------------------------------------------------------
+template <typename T>
+struct Store;
+
+template <>
+struct Store<float> {
+    static constexpr int EPV = 4;
+    static __device__ __forceinline__ void unpack(const u32x4 &v, float *f) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) f[i] = __uint_as_float(v[i]);
+    }
+    static __device__ __forceinline__ u32x4 pack(const float *f) {
+        u32x4 v;
+#pragma unroll
+        for (int i = 0; i < 4; i++) v[i] = __float_as_uint(f[i]);
+        return v;
+    }
+    static __device__ __forceinline__ float load1(const float *p) { return *p; }
+    static __device__ __forceinline__ void store1(float *p, float v) { *p = v; }
+};
+
+template <>
+struct Store<__half> {
+    static constexpr int EPV = 8;
+    static __device__ __forceinline__ void unpack(const u32x4 &v, float *f) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t w = v[i];
+            const __half2 h = *reinterpret_cast<const __half2 *>(&w);
+            const float2 t = __half22float2(h);
+            f[2 * i] = t.x;
+            f[2 * i + 1] = t.y;
+        }
+    }
+    static __device__ __forceinline__ u32x4 pack(const float *f) {
+        u32x4 v;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const __half2 h = __floats2half2_rn(f[2 * i], f[2 * i + 1]);  // round-to-nearest-even
+            v[i] = *reinterpret_cast<const uint32_t *>(&h);
+        }
+        return v;
+    }
+    static __device__ __forceinline__ float load1(const __half *p) { return __half2float(*p); }
+    static __device__ __forceinline__ void store1(__half *p, float v) { *p = __float2half_rn(v); }
+};
+
+// Streaming (read-once / write-once) 16-byte access.
+__device__ __forceinline__ u32x4 load_stream(const u32x4 *p) {
+    return __builtin_nontemporal_load(p);
+}
+__device__ __forceinline__ void store_stream(u32x4 *p, const u32x4 &v) {
+    __builtin_nontemporal_store(v, p);
+}
+
+// ---------------------------------------------------------------------------
+// Division by a launch-time constant d (n < 2^31): q = umulhi(n, mul) >> shift.
+// mul = ceil(2^(31+L) / d), shift = L-1 with L = ceil(log2 d), d >= 2; d == 1 is
+// flagged with mul == 0.  Exact for every n < 2^31 (Granlund-Montgomery).
+// ---------------------------------------------------------------------------
+struct FastDiv {
+    uint32_t mul;
+    uint32_t shift;
+    uint32_t d;
+};
+
+__device__ __forceinline__ uint32_t fast_div(uint32_t n, const FastDiv &fd) {
+    const uint32_t q = __umulhi(n, fd.mul) >> fd.shift;
+    return fd.mul == 0 ? n : q;
+}
+
+// ---------------------------------------------------------------------------
+// Wavefront reductions with DPP (no LDS traffic for the first four steps).
+// ---------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __int_as_float(
+        __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+
+constexpr int kDppXor1 = 0xB1;        // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;        // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141; // lane i <-> 7-i inside each 8
+constexpr int kDppRowMirror = 0x140;  // lane i <-> 15-i inside each 16
+
+// Sum over aligned teams of TL lanes (TL = 4, 8, 16, 32 or 64); every lane of a
+// team ends with the team total, added in the same order in every lane pair.
+template <int TL>
+__device__ __forceinline__ float team_sum(float v) {
+    static_assert(TL == 4 || TL == 8 || TL == 16 || TL == 32 || TL == 64, "team size");
+    v += dpp_move<kDppXor1>(v);
+    v += dpp_move<kDppXor2>(v);
+    if (TL >= 8) v += dpp_move<kDppHalfMirror>(v);
+    if (TL >= 16) v += dpp_move<kDppRowMirror>(v);
+    if (TL >= 32)  // swap 16-lane rows inside each 32: ds_swizzle bit mode, xor 0x10
+        v += __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401F));
+    if (TL >= 64) {
+        const float lo = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+        const float hi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+        v = lo + hi;
+    }
+    return v;
+}
+
+__device__ __forceinline__ float wave_sum(float v) { return team_sum<64>(v); }
+
+// Sum over a workgroup of NW wavefronts; `slots` is NW floats of LDS that no
+// other reduction in flight uses.  One barrier; every thread gets the total.
+template <int NW>
+__device__ __forceinline__ float block_sum(float v, float *slots) {
+    const float w = wave_sum(v);
+    if (NW == 1) return w;
+    const int tid = threadIdx.x;
+    if ((tid & (kWave - 1)) == 0) slots[tid / kWave] = w;
+    __syncthreads();
+    float t = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NW; i++) t += slots[i];
+    return t;
+}
+
+// ---------------------------------------------------------------------------
+// Activation math (float32).
+// ---------------------------------------------------------------------------
+constexpr float kLog2e = 1.44269504088896340736f;
+
+// x * 1/(1+exp(-x)); exp through the hardware 2^x, reciprocal through v_rcp_f32
+// (both about 1 ulp): relative error of the result stays below 1e-6.
+__device__ __forceinline__ float silu_f(float x) {
+    const float e = __builtin_amdgcn_exp2f(-kLog2e * x);
+    return x * __builtin_amdgcn_rcpf(1.0f + e);
+}
+
+__device__ __forceinline__ float quick_gelu_f(float x) {
+    const float e = __builtin_amdgcn_exp2f((-kLog2e * 1.702f) * x);
+    return x * __builtin_amdgcn_rcpf(1.0f + e);
+}
+
+// gelu(x) = x * Phi(x), Phi(x) = 0.5 * (1 + erf(x / sqrt 2)).
+// With t = |x| and E(t) = erfc(t / sqrt 2) = 2^(t * P(t)): Phi = 0.5 E for x < 0
+// and 1 - 0.5 E otherwise, so neither tail cancels.  P is a degree-9 weighted
+// minimax fit of log2(erfc(t / sqrt 2)) / t on (0, 5.5] (relative error of E
+// below 1.4e-7; made by fit_gelu_poly.py next to this file); its leading
+// coefficient is negative, so E -> 0 beyond the fitted range without a clamp.
+// Against float64 the result is within 3.9e-7 absolute for |x| <= 32, the same
+// as the float32 expression x * 0.5 * (1 + erff(x * sqrt 0.5)).
+__device__ __forceinline__ float gelu_erf_f(float x) {
+    const float t = fabsf(x);
+    float p = -1.824206031e-08f;
+    p = fmaf(p, t, 5.753830692e-07f);
+    p = fmaf(p, t, -7.787496543e-06f);
+    p = fmaf(p, t, 5.702746057e-05f);
+    p = fmaf(p, t, -2.093151852e-04f);
+    p = fmaf(p, t, -1.539104851e-04f);
+    p = fmaf(p, t, 7.145896088e-03f);
+    p = fmaf(p, t, -5.258353800e-02f);
+    p = fmaf(p, t, -4.591720700e-01f);
+    p = fmaf(p, t, -1.151109815e+00f);
+    const float half_e = 0.5f * __builtin_amdgcn_exp2f(p * t);
+    return x * (x < 0.0f ? half_e : 1.0f - half_e);
+}
+
+struct OpSilu {
+    static __device__ __forceinline__ float apply(float x) { return silu_f(x); }
+};
+struct OpGelu {
+    static __device__ __forceinline__ float apply(float x) { return gelu_erf_f(x); }
+};
+struct OpQuickGelu {
+    static __device__ __forceinline__ float apply(float x) { return quick_gelu_f(x); }
+};
+
+}  // namespace msd

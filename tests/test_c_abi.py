@@ -1,0 +1,77 @@
+"""CPU-side checks of the drop-in boundary: the C-ABI library loads, exports every
+symbol include/msd_hip.h declares, and its host-only entry points behave.  No
+compute call is made here (there is no GPU in the CPU test environment)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(REPO, "include", "msd_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(msd_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported(msd):
+    lib = msd.load_library()
+    declared = _declared_symbols()
+    assert len(declared) >= 14
+    for name in declared:
+        assert hasattr(lib, name), "libmsd_hip.so does not export %s" % name
+    assert sorted(msd.C_ABI_SYMBOLS) == declared  # the ctypes table covers the whole header
+
+
+def test_header_is_plain_c():
+    text = open(os.path.join(REPO, "include", "msd_hip.h")).read()
+    assert 'extern "C"' in text and "torch" not in text and "hip/hip_runtime" not in text
+    # compiles as C with no HIP headers on the include path
+    import subprocess
+    import tempfile
+    with tempfile.TemporaryDirectory() as d:
+        src = os.path.join(d, "t.c")
+        open(src, "w").write('#include "msd_hip.h"\nint main(void){return msd_ddim_timesteps(0,0,0)==-1?0:1;}\n')
+        subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-c", "-I", os.path.join(REPO, "include"),
+                        src, "-o", os.path.join(d, "t.o")], check=True)
+
+
+def test_version_and_error_strings(msd):
+    lib = msd.load_library()
+    assert lib.msd_version() >= 100
+    assert lib.msd_error_string(0) == b"ok"
+    assert b"invalid" in lib.msd_error_string(1)
+
+
+def test_ddim_timesteps_host_entry(msd, orc):
+    lib = msd.load_library()
+    for steps in (1, 2, 3, 7, 20, 25, 30, 50, 64, 100, 250, 333, 500, 999, 1000):
+        assert msd.ddim_timesteps(steps) == orc.ddim_timesteps(steps), steps
+    assert msd.ddim_timesteps(50)[-1] == 981
+    assert lib.msd_ddim_timesteps(0, None, 0) == -1
+    assert lib.msd_ddim_timesteps(1001, None, 0) == -1
+    # cap smaller than the list: count is still returned, nothing past cap is written
+    buf = (ctypes.c_int * 4)(-7, -7, -7, -7)
+    assert lib.msd_ddim_timesteps(50, buf, 3) == 50
+    assert list(buf) == [1, 21, 41, -7]
+    with pytest.raises(msd.MsdError):
+        msd.ddim_timesteps(0)
+
+
+def test_argument_validation_needs_no_gpu(msd):
+    lib = msd.load_library()
+    # rejected before any HIP call
+    assert lib.msd_groupnorm(None, None, None, None, 1, 30, 16, 32, 1e-5, 0, 0, None) == 1
+    assert lib.msd_groupnorm(None, None, None, None, 1, 32, 16, 0, 1e-5, 0, 0, None) == 1
+    assert lib.msd_layernorm(None, None, None, None, 4, 64, 1e-5, 0, None) == 1
+    assert lib.msd_geglu(None, None, 4, 64, 0, None) == 1
+    assert lib.msd_silu(None, None, 4, 0, None) == 1
+    assert lib.msd_timestep_embedding(None, None, 2, 321, 10000.0, 0, None) == 1
+    assert lib.msd_set_groupnorm_target_blocks(0) == 1
+
+
+def test_missing_library_fails_loudly(msd):
+    with pytest.raises(msd.MsdError):
+        msd.load_library(os.path.join(REPO, "does_not_exist.so"))

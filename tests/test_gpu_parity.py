@@ -1,0 +1,319 @@
+"""Parity of the HIP kernels (through the C ABI) against the CPU oracle.
+
+Same seeded inputs go to the oracle (float32 restatement of the reference's
+kernels) and to the GPU.  fp32 storage: 1e-5 relative; fp16 storage: the oracle
+runs on fp16-rounded inputs and its output is rounded to fp16 (see
+tolerances.py).  Shapes are the reference's SD UNet / text-encoder shapes at
+batch 2 plus the edge cases the reference's preconditions and the kernels'
+dispatch split on.
+"""
+import numpy as np
+import pytest
+
+from tolerances import assert_close_f16, assert_close_f32
+
+pytestmark = pytest.mark.gpu
+
+# (channels, height*width) of every GroupNorm in one UNet step; in-norm and out-norm
+# of the 22 ResBlocks (M/UNetModel.cpp:86-1018) and the final norm (:1007)
+UNET_GN_SHAPES = sorted({
+    (320, 4096), (640, 4096), (960, 4096), (320, 1024), (640, 1024), (1280, 1024), (960, 1024),
+    (1920, 1024), (640, 256), (1280, 256), (1920, 256), (2560, 256), (1280, 64), (2560, 64),
+})
+CFG2_SHAPES = [(320, 4096, 2001), (640, 1024, 2002), (1280, 256, 2003), (1280, 64, 2004),
+               (960, 1024, 2005), (1920, 256, 2006)]
+
+
+def _torch():
+    import torch
+    return torch
+
+
+def _to_dev(a, cuda, half=False):
+    torch = _torch()
+    t = torch.from_numpy(np.ascontiguousarray(a)).to(cuda)
+    return t.half() if half else t
+
+
+def _affine(orc, channels, seed):
+    return (orc.normal((channels,), seed=seed + 500000, mean=1.0, sigma=0.1),
+            orc.normal((channels,), seed=seed + 600000, mean=0.0, sigma=0.1))
+
+
+def _run_groupnorm(msd, orc, cuda, x, g, b, groups, eps, silu, half, inplace=False):
+    xin = orc.round_to_half(x) if half else x
+    ref = orc.groupnorm(xin, g, b, groups, eps, silu)
+    xd = _to_dev(xin, cuda, half)
+    out = msd.groupnorm(xd, _to_dev(g, cuda), _to_dev(b, cuda), groups, eps, silu,
+                        out=xd if inplace else None)
+    got = out.float().cpu().numpy()
+    if half:
+        return assert_close_f16(got, orc.round_to_half(ref), "groupnorm f16 %s" % (x.shape,))
+    return assert_close_f32(got, ref, what="groupnorm f32 %s" % (x.shape,)), None
+
+
+# ----------------------------------------------------------------- GroupNorm
+def test_config1_groupnorm_silu_fp32(msd, orc, cuda):
+    x = orc.normal((1, 320, 64, 64), seed=1001)
+    g, b = _affine(orc, 320, 1001)
+    _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half=False)
+    assert msd.status() == 0
+
+
+@pytest.mark.parametrize("half", [False, True], ids=["f32", "f16"])
+@pytest.mark.parametrize("channels,hw,seed", CFG2_SHAPES)
+def test_config2_groupnorm_silu_sweep(msd, orc, cuda, channels, hw, seed, half):
+    side = int(round(hw ** 0.5))
+    x = orc.normal((2, channels, side, side), seed=seed, sigma=2.0)
+    g, b = _affine(orc, channels, seed)
+    worst, exact = _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half)
+    if half:
+        assert exact > 0.99  # nearly every element is bit-identical to the rounded oracle
+    assert msd.status() == 0
+
+
+@pytest.mark.parametrize("channels,hw", UNET_GN_SHAPES)
+def test_unet_step_groupnorm_shapes_fp16(msd, orc, cuda, channels, hw):
+    x = orc.normal((2, channels, hw), seed=5001 + channels + hw, sigma=1.5, mean=0.2)
+    g, b = _affine(orc, channels, 5001 + channels)
+    _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half=True)
+
+
+@pytest.mark.parametrize("half", [False, True], ids=["f32", "f16"])
+def test_groupnorm_in_place_and_no_silu(msd, orc, cuda, half):
+    # in place as at M/nn/ResBlock.cpp:222; eps 1e-6 without SiLU as in SpatialTransformer
+    x = orc.normal((2, 640, 32, 32), seed=77, sigma=1.0, mean=-0.5)
+    g, b = _affine(orc, 640, 77)
+    _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half, inplace=True)
+    _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-6, False, half, inplace=True)
+    _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-6, False, half)
+
+
+@pytest.mark.parametrize("target_blocks", [1, 64, 2048, 8192])
+def test_groupnorm_every_split_factor(msd, orc, cuda, target_blocks):
+    # the same tensor through 1 .. 64 workgroups per group must agree with the oracle
+    lib = msd.load_library()
+    x = orc.normal((2, 320, 64, 64), seed=88, sigma=2.0, mean=1.0)
+    g, b = _affine(orc, 320, 88)
+    try:
+        assert lib.msd_set_groupnorm_target_blocks(target_blocks) == 0
+        for half in (False, True):
+            _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half)
+    finally:
+        lib.msd_set_groupnorm_target_blocks(512)
+    assert msd.status() == 0
+
+
+def test_groupnorm_repeated_launches_reuse_scratch(msd, orc, cuda):
+    # the arrival counters are never reset: many launches with changing split factors
+    shapes = [(2, 320, 4096), (2, 1280, 64), (1, 640, 1024), (2, 1920, 256), (2, 320, 4096)]
+    for rep in range(3):
+        for i, shp in enumerate(shapes):
+            x = orc.normal(shp, seed=900 + i + 10 * rep, sigma=2.0)
+            g, b = _affine(orc, shp[1], 900 + i)
+            _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half=True)
+    assert msd.status() == 0
+
+
+@pytest.mark.parametrize("shape,groups", [
+    ((1, 32, 3, 3), 32),      # hw not a multiple of the vector width: scalar kernel
+    ((3, 64, 5, 7), 8),       # odd everything
+    ((2, 64, 2, 4), 32),      # one 16-byte vector per channel (fp16)
+    ((1, 96, 24, 24), 32),    # ragged slices: 3 channels per group
+    ((5, 32, 40, 40), 4),     # few large groups, odd batch
+    ((1, 4, 512, 512), 1),    # one huge group: maximum split
+])
+@pytest.mark.parametrize("half", [False, True], ids=["f32", "f16"])
+def test_groupnorm_edge_shapes(msd, orc, cuda, shape, groups, half):
+    x = orc.normal(shape, seed=sum(shape), sigma=1.3, mean=0.1)
+    xin = orc.round_to_half(x) if half else x
+    g, b = _affine(orc, shape[1], 31)
+    ref = orc.groupnorm64(xin, g, b, groups, 1e-5, True)  # textbook: these shapes break the
+    xd = _to_dev(xin, cuda, half)                         # reference's % 64 precondition
+    got = msd.groupnorm(xd, _to_dev(g, cuda), _to_dev(b, cuda), groups, 1e-5, True).float().cpu().numpy()
+    if half:
+        assert_close_f16(got, orc.round_to_half(ref.astype(np.float32)), "gn edge f16")
+    else:
+        assert_close_f32(got, ref, what="gn edge f32")
+    assert msd.status() == 0
+
+
+def test_groupnorm_misaligned_and_empty(msd, orc, cuda):
+    torch = _torch()
+    x = orc.normal((1, 64, 8, 8), seed=5)
+    g, b = _affine(orc, 64, 5)
+    ref = orc.groupnorm(x, g, b, 32, 1e-5, True)
+    buf = torch.zeros(x.size + 1, device=cuda)
+    buf[1:] = torch.from_numpy(x.reshape(-1)).to(cuda)
+    xin = buf[1:].view(1, 64, 8, 8)  # 4-byte aligned only
+    got = msd.groupnorm(xin, _to_dev(g, cuda), _to_dev(b, cuda), 32, 1e-5, True).cpu().numpy()
+    assert_close_f32(got, ref, what="gn misaligned")
+    empty = torch.empty((0, 64, 8, 8), device=cuda)
+    assert msd.groupnorm(empty, _to_dev(g, cuda), _to_dev(b, cuda), 32).numel() == 0
+    lib = msd.load_library()
+    assert lib.msd_groupnorm(None, None, None, None, 1, 30, 16, 32, 1e-5, 0, 0, None) == 1
+    assert lib.msd_groupnorm(None, None, None, None, 1, 32, 16, 32, 1e-5, 0, 7, None) == 1
+
+
+def test_groupnorm_statistics_property_full_size(msd, orc, cuda):
+    # size-independent check at the largest UNet shape: unit statistics per (sample, group)
+    torch = _torch()
+    x = torch.randn((2, 960, 64, 64), device=cuda, generator=torch.Generator(device=cuda).manual_seed(3)) * 3 + 1
+    one, zero = torch.ones(960, device=cuda), torch.zeros(960, device=cuda)
+    y = msd.groupnorm(x, one, zero, 32, 1e-5, False).double().view(2, 32, -1)
+    assert y.mean(dim=2).abs().max().item() < 1e-5
+    assert (y.var(dim=2, unbiased=False) - 1.0).abs().max().item() < 1e-4
+    # affine linearity: GN(x; g, b) == g * GN(x; 1, 0) + b
+    g = torch.rand(960, device=cuda) + 0.5
+    b = torch.randn(960, device=cuda)
+    y2 = msd.groupnorm(x, g, b, 32, 1e-5, False)
+    base = msd.groupnorm(x, one, zero, 32, 1e-5, False)
+    assert (y2 - (base * g.view(1, -1, 1, 1) + b.view(1, -1, 1, 1))).abs().max().item() < 1e-5
+    assert msd.status() == 0
+
+
+def test_groupnorm_golden_fixtures(msd, golden, cuda):
+    for name in ("gn_a", "gn_b", "gn_c"):
+        x, g, b = (_to_dev(golden[name + k], cuda) for k in ("_x", "_gamma", "_beta"))
+        eps = float(golden[name + "_eps"])
+        assert_close_f32(msd.groupnorm(x, g, b, 32, eps, False).cpu().numpy(), golden[name + "_y"], what=name)
+        assert_close_f32(msd.groupnorm(x, g, b, 32, eps, True).cpu().numpy(), golden[name + "_y_silu"], what=name)
+
+
+# ----------------------------------------------------------------- LayerNorm
+@pytest.mark.parametrize("rows,dim,seed", [(8192, 320, 3001), (2048, 640, 3002), (512, 1280, 3003),
+                                           (128, 1280, 3007)])
+def test_config3_layernorm_fp16(msd, orc, cuda, rows, dim, seed):
+    x = orc.round_to_half(orc.normal((2, rows // 2, dim), seed=seed))
+    g, b = _affine(orc, dim, seed)
+    ref = orc.round_to_half(orc.layernorm(x, g, b, 1e-5))
+    got = msd.layernorm(_to_dev(x, cuda, True), _to_dev(g, cuda), _to_dev(b, cuda)).float().cpu().numpy()
+    worst, exact = assert_close_f16(got, ref, "layernorm f16 %dx%d" % (rows, dim))
+    assert exact > 0.99
+
+
+@pytest.mark.parametrize("rows,dim,seed", [(77, 768, 4001), (154, 768, 4002), (77, 1024, 4004)])
+def test_config4_layernorm_fp32_outliers(msd, orc, cuda, rows, dim, seed):
+    x = orc.add_outliers(orc.normal((rows, dim), seed=seed), seed=seed)
+    g, b = _affine(orc, dim, seed)
+    got = msd.layernorm(_to_dev(x, cuda), _to_dev(g, cuda), _to_dev(b, cuda)).cpu().numpy()
+    assert_close_f32(got, orc.layernorm(x, g, b, 1e-5), what="layernorm f32 outliers")
+
+
+@pytest.mark.parametrize("half", [False, True], ids=["f32", "f16"])
+@pytest.mark.parametrize("rows,dim", [(1, 64), (3, 128), (5, 192), (9, 320), (33, 448), (7, 576),
+                                      (4, 2048), (3, 4096), (2, 8192), (5, 100), (6, 36), (2, 7),
+                                      (3, 6400)])
+def test_layernorm_dims_and_ragged_rows(msd, orc, cuda, rows, dim, half):
+    # every team width / vectors-per-lane pairing, the scalar kernel (dim 100, 36, 7) and
+    # row counts that do not fill the last wavefront
+    x = orc.normal((rows, dim), seed=rows * 1000 + dim, sigma=2.0, mean=3.0)
+    xin = orc.round_to_half(x) if half else x
+    g, b = _affine(orc, dim, dim)
+    ref = orc.layernorm64(xin, g, b, 1e-5)
+    got = msd.layernorm(_to_dev(xin, cuda, half), _to_dev(g, cuda), _to_dev(b, cuda)).float().cpu().numpy()
+    if half:
+        assert_close_f16(got, orc.round_to_half(ref.astype(np.float32)), "ln dims f16")
+    else:
+        assert_close_f32(got, ref, what="ln dims f32")
+
+
+def test_layernorm_in_place_fixtures_and_empty(msd, orc, golden, cuda):
+    torch = _torch()
+    for name in ("ln_a", "ln_b", "ln_c", "ln_d"):
+        x, g, b = (_to_dev(golden[name + k], cuda) for k in ("_x", "_gamma", "_beta"))
+        y = msd.layernorm(x, g, b, float(golden[name + "_eps"]), out=x)  # in place
+        assert_close_f32(y.cpu().numpy(), golden[name + "_y"], what=name)
+    e = torch.empty((0, 320), device=cuda)
+    assert msd.layernorm(e, torch.ones(320, device=cuda), torch.zeros(320, device=cuda)).numel() == 0
+
+
+# ----------------------------------------------------------------- GEGLU and activations
+@pytest.mark.parametrize("rows,inner,seed", [(8192, 1280, 3004), (2048, 2560, 3005), (512, 5120, 3006),
+                                             (128, 5120, 3008)])
+def test_config3_geglu_fp16(msd, orc, cuda, rows, inner, seed):
+    proj = orc.round_to_half(orc.normal((rows, 2 * inner), seed=seed))
+    ref = orc.round_to_half(orc.geglu(proj))
+    got = msd.geglu(_to_dev(proj, cuda, True)).float().cpu().numpy()
+    worst, exact = assert_close_f16(got, ref, "geglu f16 %dx%d" % (rows, inner))
+    assert exact > 0.99
+
+
+@pytest.mark.parametrize("rows,inner", [(77, 1280), (5, 64), (3, 20), (7, 9), (1025, 8), (1, 1)])
+@pytest.mark.parametrize("half", [False, True], ids=["f32", "f16"])
+def test_geglu_shapes_fp32_fp16(msd, orc, golden, cuda, rows, inner, half):
+    proj = orc.normal((rows, 2 * inner), seed=rows + inner, sigma=2.5)
+    pin = orc.round_to_half(proj) if half else proj
+    ref = orc.geglu(pin)
+    got = msd.geglu(_to_dev(pin, cuda, half)).float().cpu().numpy()
+    if half:
+        assert_close_f16(got, orc.round_to_half(ref), "geglu shapes f16")
+    else:
+        assert_close_f32(got, ref, what="geglu shapes f32")
+        assert_close_f32(msd.geglu(_to_dev(golden["geglu_proj"], cuda)).cpu().numpy(), golden["geglu_y"])
+
+
+@pytest.mark.parametrize("name", ["silu", "gelu", "quick_gelu"])
+@pytest.mark.parametrize("half", [False, True], ids=["f32", "f16"])
+def test_activations(msd, orc, golden, cuda, name, half):
+    fn, ref_fn = getattr(msd, name), getattr(orc, name)
+    cases = [orc.normal((2, 77, 3072), seed=4003),               # config 4 MLP hidden
+             orc.add_outliers(orc.normal((77, 4096), seed=4005), seed=4005),  # the reference's size
+             orc.normal((2, 1280), seed=5002),                   # SiLU on the time embedding
+             golden["act_x"], orc.normal((1031,), seed=9, sigma=4.0), orc.normal((3,), seed=10)]
+    for x in cases:
+        xin = orc.round_to_half(x) if half else np.ascontiguousarray(x)
+        xd = _to_dev(xin, cuda, half)
+        got = fn(xd, out=xd).float().cpu().numpy()  # in place, like every reference call site
+        if half:
+            assert_close_f16(got, orc.round_to_half(ref_fn(xin)), name + " f16")
+        else:
+            assert_close_f32(got, ref_fn(xin), what=name + " f32")
+    if not half:
+        got = fn(_to_dev(golden["act_x"], cuda)).cpu().numpy()
+        assert_close_f32(got, golden["act_" + name], what=name + " fixture")
+
+
+def test_activation_special_values(msd, cuda):
+    torch = _torch()
+    x = torch.tensor([0.0, -0.0, 100.0, -100.0, 1e-30, -1e-30, 88.0, -88.0, 30.0, -30.0], device=cuda)
+    s = msd.silu(x).cpu().numpy()
+    assert s[0] == 0 and s[2] == 100.0 and abs(s[3]) < 1e-30 and s[8] == 30.0
+    ge = msd.gelu(x).cpu().numpy()
+    assert ge[0] == 0 and ge[2] == 100.0 and abs(ge[3]) < 1e-30 and ge[6] == 88.0 and abs(ge[9]) < 1e-30
+    assert np.isfinite(s).all() and np.isfinite(ge).all()
+
+
+# ----------------------------------------------------------------- timestep embedding + DDIM list
+def test_timestep_embedding_all_timesteps(msd, orc, golden, cuda):
+    torch = _torch()
+    ts = np.arange(0, 1000, dtype=np.int64)
+    got = msd.timestep_embedding(torch.from_numpy(ts).to(cuda), 320).cpu().numpy()
+    ref = np.stack([orc.timestep_embedding(int(t)) for t in ts])
+    assert_close_f32(got, ref, what="timestep embedding")
+    assert (got == ref).mean() > 0.95  # same frequencies and angles; cos/sin differ by <= 1 ulp
+    # t = 0 row is exactly [1.. | 0..]; column 0 is cos(t), sin(t)
+    assert np.array_equal(got[0], np.concatenate([np.ones(160), np.zeros(160)]).astype(np.float32))
+    k = golden["temb_t"]
+    g2 = msd.timestep_embedding(torch.from_numpy(k).to(cuda), 320).cpu().numpy()
+    assert np.abs(g2 - golden["temb_f64"]).max() < 1.3e-4  # |t| * ulp(freq) at t ~ 1000
+    # fp16 storage and another dim / period
+    h = msd.timestep_embedding(torch.from_numpy(ts[:64]).to(cuda), 320, dtype=torch.float16).float().cpu().numpy()
+    assert_close_f16(h, orc.round_to_half(ref[:64]), "temb f16")
+    o = msd.timestep_embedding(torch.tensor([13], device=cuda), 64, max_period=100.0).cpu().numpy()[0]
+    assert_close_f32(o, orc.timestep_embedding(13, 64, 100.0))
+
+
+def test_config5_timesteps_feed_embedding_bit_exact_integers(msd, orc, cuda):
+    torch = _torch()
+    for steps in (50, 25, 30, 1000, 1):
+        assert msd.ddim_timesteps(steps) == orc.ddim_timesteps(steps)
+    sched = msd.ddim_timesteps(25)[::-1]  # the sampler walks the list from the back
+    assert sched[0] == 961 and sched[-1] == 1
+    t = torch.tensor(sched, dtype=torch.int64, device=cuda)
+    emb = msd.timestep_embedding(t, 320).cpu().numpy()
+    ref = np.stack([orc.timestep_embedding(s) for s in sched])
+    assert_close_f32(emb, ref)
+    rnd = orc.uniform_int(2, 5001, 0, 999)
+    emb2 = msd.timestep_embedding(torch.from_numpy(rnd).to(cuda), 320, dtype=torch.float16)
+    assert emb2.shape == (2, 320)
