@@ -1,0 +1,386 @@
+#!/usr/bin/env python3
+"""Benchmark of the norm / activation / embedding path on one MI355X.
+
+A "step" is one UNet step's worth of the hot path at batch 2 (CFG), fp16 storage:
+the timestep embedding, 23 SiLU(emb), 45 GroupNorm(32)+SiLU (in- and out-norm of the
+22 ResBlocks plus the final norm), 48 LayerNorms and 16 GEGLUs at their real shapes,
+each layer on its own HBM-resident buffers, launched back to back on one stream.
+`value` = algorithmic bytes of one step / time per step.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode graph|eager]
+                    [--no-cpu] [--no-shapes]
+
+Prints ONE JSON line (see the keys below).  The CPU oracle is used only for the
+`cpu_baseline` leg.
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+REPO = os.path.dirname(os.path.abspath(__file__))
+if REPO not in sys.path:
+    sys.path.insert(0, REPO)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+# ----------------------------------------------------------------------------
+# The per-step workload (call order of UNetModel::forward, M/UNetModel.cpp:1078-1929)
+# ----------------------------------------------------------------------------
+# ResBlocks: (in_channels, out_channels, side) in execution order
+RESBLOCKS = (
+    [(320, 320, 64)] * 2 + [(320, 640, 32), (640, 640, 32), (640, 1280, 16), (1280, 1280, 16)] +
+    [(1280, 1280, 8)] * 2 +                       # input blocks 10, 11
+    [(1280, 1280, 8)] * 2 +                       # middle block
+    [(2560, 1280, 8)] * 3 + [(2560, 1280, 16)] * 2 + [(1920, 1280, 16)] +
+    [(1920, 640, 32), (1280, 640, 32), (960, 640, 32)] +
+    [(960, 320, 64), (640, 320, 64), (640, 320, 64)]
+)
+# transformer blocks: (dim, tokens); 3 LayerNorms and 1 GEGLU each
+TRANSFORMERS = [(320, 4096)] * 2 + [(640, 1024)] * 2 + [(1280, 256)] * 2 + [(1280, 64)] + \
+               [(1280, 256)] * 3 + [(640, 1024)] * 3 + [(320, 4096)] * 3
+BATCH = 2
+ELT = 2  # fp16 storage
+
+
+def step_layers():
+    """List of (kind, params) in execution order for one UNet step."""
+    layers = [("temb", {"dim": 320}), ("silu", {"n": BATCH * 1280})]  # time_embed MLP's SiLU
+    tr = iter(TRANSFORMERS)
+    # which ResBlocks are followed by a SpatialTransformer (M/UNetModel.cpp:86-1018)
+    followed = [True, True, True, True, True, True, False, False,  # input blocks 1,2,4,5,7,8,10,11
+                True, False,                                         # middle: res, ST, res
+                False, False, False, True, True, True,               # output 0..5
+                True, True, True, True, True, True]                  # output 6..11
+    assert len(followed) == len(RESBLOCKS) == 22 and sum(followed) == 16
+    for (cin, cout, side), st in zip(RESBLOCKS, followed):
+        layers.append(("gn_silu", {"c": cin, "hw": side * side, "inplace": False}))
+        layers.append(("silu", {"n": BATCH * 1280}))  # SiLU(emb) before the ResBlock's Linear
+        layers.append(("gn_silu", {"c": cout, "hw": side * side, "inplace": True}))
+        if st:
+            dim, tokens = next(tr)
+            assert tokens == side * side
+            for _ in range(3):
+                layers.append(("ln", {"rows": BATCH * tokens, "dim": dim}))
+            layers.append(("geglu", {"rows": BATCH * tokens, "inner": 4 * dim}))
+    layers.append(("gn_silu", {"c": 320, "hw": 4096, "inplace": True}))  # final norm + SiLU
+    return layers
+
+
+def layer_bytes(kind, p):
+    """Algorithmic HBM bytes of one launch (gamma/beta excluded, as in the baseline table)."""
+    if kind == "gn_silu":
+        return 2 * BATCH * p["c"] * p["hw"] * ELT
+    if kind == "ln":
+        return 2 * p["rows"] * p["dim"] * ELT
+    if kind == "geglu":
+        return 3 * p["rows"] * p["inner"] * ELT
+    return 0  # temb / SiLU(emb): a few KB, launch-bound, not counted
+
+
+class Step:
+    """Device buffers and launch closures for one step."""
+
+    def __init__(self, msd, torch, dev, seed=5001):
+        self.msd, self.torch = msd, torch
+        g = torch.Generator(device=dev).manual_seed(seed)
+        self.launches = []
+        self.bytes = 0
+        self.by_kind = {}
+        lib = msd.load_library()
+        import ctypes
+        vp = ctypes.c_void_p
+        self._keep = []
+
+        def randn(*shape, dtype=torch.float16):
+            t = torch.randn(*shape, device=dev, dtype=torch.float32, generator=g).to(dtype)
+            self._keep.append(t)
+            return t
+
+        # integer timesteps, uniform in [0, 999]
+        self.t = torch.randint(0, 1000, (BATCH,), device=dev, dtype=torch.int64, generator=g)
+        self._keep.append(self.t)
+        affine = {}
+
+        def gb(c):
+            if c not in affine:
+                affine[c] = (1.0 + 0.1 * randn(c, dtype=torch.float32), 0.1 * randn(c, dtype=torch.float32))
+                self._keep.extend(affine[c])
+            return affine[c]
+
+        for kind, p in step_layers():
+            nb = layer_bytes(kind, p)
+            self.bytes += nb
+            k = self.by_kind.setdefault(kind, {"launches": 0, "bytes": 0})
+            k["launches"] += 1
+            k["bytes"] += nb
+            if kind == "temb":
+                out = torch.empty((BATCH, p["dim"]), device=dev, dtype=torch.float16)
+                self._keep.append(out)
+                args = (vp(self.t.data_ptr()), vp(out.data_ptr()), BATCH, p["dim"], 10000.0, msd.DTYPE_F16)
+                fn = lib.msd_timestep_embedding
+            elif kind == "silu":
+                x = randn(p["n"])
+                args = (vp(x.data_ptr()), vp(x.data_ptr()), p["n"], msd.DTYPE_F16)
+                fn = lib.msd_silu
+            elif kind == "gn_silu":
+                x = randn(BATCH, p["c"], p["hw"]) * 2.0
+                self._keep.append(x)
+                y = x if p["inplace"] else torch.empty_like(x)
+                self._keep.append(y)
+                ga, be = gb(p["c"])
+                args = (vp(x.data_ptr()), vp(y.data_ptr()), vp(ga.data_ptr()), vp(be.data_ptr()), BATCH,
+                        p["c"], p["hw"], 32, 1e-5, 1, msd.DTYPE_F16)
+                fn = lib.msd_groupnorm
+            elif kind == "ln":
+                x = randn(p["rows"], p["dim"])
+                y = torch.empty_like(x)
+                self._keep.append(y)
+                ga, be = gb(p["dim"])
+                args = (vp(x.data_ptr()), vp(y.data_ptr()), vp(ga.data_ptr()), vp(be.data_ptr()), p["rows"],
+                        p["dim"], 1e-5, msd.DTYPE_F16)
+                fn = lib.msd_layernorm
+            elif kind == "geglu":
+                x = randn(p["rows"], 2 * p["inner"])
+                y = torch.empty((p["rows"], p["inner"]), device=dev, dtype=torch.float16)
+                self._keep.append(y)
+                args = (vp(x.data_ptr()), vp(y.data_ptr()), p["rows"], p["inner"], msd.DTYPE_F16)
+                fn = lib.msd_geglu
+            else:
+                raise AssertionError(kind)
+            self.launches.append((kind, fn, args))
+
+    def run(self, stream_ptr, only=None):
+        for kind, fn, args in self.launches:
+            if only is None or kind == only:
+                rc = fn(*args, stream_ptr)
+                if rc != 0:
+                    raise RuntimeError("%s failed: %d" % (kind, rc))
+
+
+def timed_replays(torch, fn, reps):
+    """Wall time (s) of `reps` calls of fn, bracketed by device synchronisation."""
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        fn()
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0
+
+
+def event_time_ms(torch, fn, reps):
+    """Elapsed GPU time (ms) of `reps` calls of fn between two HIP events recorded on
+    the stream the kernels are launched on (torch's current stream)."""
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    a.record()
+    for _ in range(reps):
+        fn()
+    b.record()
+    b.synchronize()
+    return a.elapsed_time(b)
+
+
+def capture(torch, msd, stream, body):
+    """Captures body() (launches on the current stream) into a HIP graph; returns replay()."""
+    import ctypes
+    with torch.cuda.stream(stream):
+        msd.check(msd.load_library().msd_init(ctypes.c_void_p(stream.cuda_stream)))  # scratch before capture
+        body()  # warm: module load, scratch
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        body()
+    torch.cuda.synchronize()
+    return graph.replay
+
+
+def shape_table(torch, msd, dev, stream):
+    """Per-kernel µs / GB/s / % of HBM peak at the UNet shapes, fp16 and fp32, each launch on
+    its own buffers (rotating over > 600 MB so nothing is cache-resident), graph-replayed."""
+    import ctypes
+    vp = ctypes.c_void_p
+    lib = msd.load_library()
+    rows = []
+    cases = []
+    for c, side in [(320, 64), (640, 32), (1280, 16), (1280, 8), (960, 32), (1920, 16)]:
+        cases.append(("groupnorm_silu", {"c": c, "hw": side * side}))
+    for r, d in [(8192, 320), (2048, 640), (512, 1280)]:
+        cases.append(("layernorm", {"rows": r, "dim": d}))
+    for r, i in [(8192, 1280), (2048, 2560), (512, 5120)]:
+        cases.append(("geglu", {"rows": r, "inner": i}))
+    for kind, p in cases:
+        for dt, code, elt in ((torch.float16, msd.DTYPE_F16, 2), (torch.float32, msd.DTYPE_F32, 4)):
+            if kind != "groupnorm_silu" and dt == torch.float32:
+                continue
+            if kind == "groupnorm_silu":
+                n_in = n_out = BATCH * p["c"] * p["hw"]
+                nbytes = 2 * n_in * elt
+            elif kind == "layernorm":
+                n_in = n_out = p["rows"] * p["dim"]
+                nbytes = 2 * n_in * elt
+            else:
+                n_in, n_out = 2 * p["rows"] * p["inner"], p["rows"] * p["inner"]
+                nbytes = 3 * n_out * elt
+            copies = max(4, min(256, int(640e6 // nbytes) + 1))
+            xs = [torch.randn(n_in, device=dev, dtype=torch.float32).to(dt) for _ in range(copies)]
+            ys = [torch.empty(n_out, device=dev, dtype=dt) for _ in range(copies)]
+            cdim = p.get("c", p.get("dim", 1))
+            ga = torch.ones(cdim, device=dev)
+            be = torch.zeros(cdim, device=dev)
+
+            def body():
+                sp = vp(torch.cuda.current_stream().cuda_stream)
+                for x, y in zip(xs, ys):
+                    if kind == "groupnorm_silu":
+                        rc = lib.msd_groupnorm(vp(x.data_ptr()), vp(y.data_ptr()), vp(ga.data_ptr()),
+                                               vp(be.data_ptr()), BATCH, p["c"], p["hw"], 32, 1e-5, 1, code, sp)
+                    elif kind == "layernorm":
+                        rc = lib.msd_layernorm(vp(x.data_ptr()), vp(y.data_ptr()), vp(ga.data_ptr()),
+                                               vp(be.data_ptr()), p["rows"], p["dim"], 1e-5, code, sp)
+                    else:
+                        rc = lib.msd_geglu(vp(x.data_ptr()), vp(y.data_ptr()), p["rows"], p["inner"], code, sp)
+                    assert rc == 0
+            replay = capture(torch, msd, stream, body)
+            with torch.cuda.stream(stream):
+                replay()
+                reps = max(2, int(2000 // copies))
+                ms = event_time_ms(torch, replay, reps)
+            us = ms * 1e3 / (reps * copies)
+            gbs = nbytes / us / 1e3
+            rows.append({"kernel": kind, "shape": p, "dtype": "f16" if elt == 2 else "f32",
+                         "bytes": nbytes, "us": round(us, 3), "GBps": round(gbs, 1),
+                         "pct_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 1)})
+            del xs, ys
+            torch.cuda.empty_cache()
+    return rows
+
+
+def cpu_baseline(total_bytes):
+    """The reference path as host loops (the CPU oracle, fp32, unfused passes exactly as the
+    reference enqueues them) over one full step, timed on this host's cores."""
+    import numpy as np
+    from oracle import pyoracle as orc
+    threads = orc.max_threads()
+    t_total = 0.0
+    for kind, p in step_layers():
+        if kind == "gn_silu":
+            x = orc.normal((BATCH, p["c"], p["hw"]), seed=p["c"] + p["hw"], sigma=2.0)
+            g, b = np.ones(p["c"], np.float32), np.zeros(p["c"], np.float32)
+            t0 = time.perf_counter()
+            orc.groupnorm(x, g, b, 32, 1e-5, silu=True)
+        elif kind == "ln":
+            x = orc.normal((p["rows"], p["dim"]), seed=p["rows"] + p["dim"])
+            g, b = np.ones(p["dim"], np.float32), np.zeros(p["dim"], np.float32)
+            t0 = time.perf_counter()
+            orc.layernorm(x, g, b, 1e-5)
+        elif kind == "geglu":
+            x = orc.normal((p["rows"], 2 * p["inner"]), seed=p["rows"] + p["inner"])
+            t0 = time.perf_counter()
+            orc.geglu(x)
+        elif kind == "silu":
+            x = orc.normal((p["n"],), seed=1)
+            t0 = time.perf_counter()
+            orc.silu(x)
+        else:
+            t0 = time.perf_counter()
+            for t in (17, 801):
+                orc.timestep_embedding(t)
+        t_total += time.perf_counter() - t0
+    return {"value": round(total_bytes / t_total / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "ms_per_step": round(t_total * 1e3, 2),
+            "sample": "one full UNet step (45 GN+SiLU, 48 LN, 16 GEGLU, 23 SiLU, 1 embedding) in fp32, "
+                      "unfused passes as the reference enqueues them, OpenMP over groups/rows; "
+                      "GB/s uses the same fp16 algorithmic bytes as the GPU figure"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--mode", choices=["graph", "eager"], default="graph")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-shapes", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no cross-GPU step and the build uses a single "
+              "device; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import ctypes
+    import torch
+    msd = importlib.import_module("mobile-stable-diffusion_amd")
+    msd.load_library()  # raises if the HIP library is not built
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.Stream()
+    step = Step(msd, torch, dev)
+
+    def eager_step():
+        step.run(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+
+    with torch.cuda.stream(stream):
+        if args.mode == "graph":
+            run_step = capture(torch, msd, stream, eager_step)
+        else:
+            msd.init()
+            run_step = eager_step
+        for _ in range(args.warmup):
+            run_step()
+        seconds = timed_replays(torch, run_step, args.steps)
+        assert msd.status() == 0
+        ms_per_step = seconds * 1e3 / args.steps
+        value = step.bytes / (seconds / args.steps) / 1e9
+
+        # per-kernel-family timing inside the same step order (HIP events on the launch stream)
+        families = {}
+        for kind in ("gn_silu", "ln", "geglu"):
+            def fam(kind=kind):
+                step.run(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream), only=kind)
+            replay = capture(torch, msd, stream, fam) if args.mode == "graph" else fam
+            for _ in range(3):
+                replay()
+            reps = max(5, args.steps // 4)
+            ms = event_time_ms(torch, replay, reps) / reps
+            k = step.by_kind[kind]
+            gbs = k["bytes"] / ms / 1e6
+            families[kind] = {"launches": k["launches"], "bytes": k["bytes"], "us_total": round(ms * 1e3, 2),
+                              "us_per_launch": round(ms * 1e3 / k["launches"], 3), "GBps": round(gbs, 1),
+                              "pct_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 1)}
+
+    dominant = max(families, key=lambda k: families[k]["us_total"])
+    kernel_names = {"gn_silu": "gn_split_kernel<__half,K,SILU>", "ln": "ln_team_kernel<__half,VPL,TL>",
+                    "geglu": "geglu_kernel<__half>"}
+    dk = families[dominant]
+    roofline = {"bound": "hbm", "kernel": kernel_names[dominant], "achieved": dk["GBps"], "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": round(dk["GBps"] / HBM_PEAK_GBS, 4),
+                "bytes_per_launch": dk["bytes"] // dk["launches"], "us_per_launch": dk["us_per_launch"],
+                "traffic": None}
+
+    out = {
+        "metric": "fused GroupNorm+SiLU/LayerNorm/GEGLU HBM GB/s over one SD UNet step (batch 2, fp16 storage)",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "unet_step_norm_act: 45 GroupNorm(32)+SiLU, 48 LayerNorm, 16 GEGLU, 23 SiLU(emb), "
+                               "1 timestep embedding at SD UNet shapes, batch 2, fp16 storage / fp32 arithmetic",
+                   "bytes_per_step": step.bytes, "launches_per_step": len(step.launches), "launch_mode": args.mode,
+                   "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 1)},
+        "roofline": roofline,
+        "kernel_families": families,
+    }
+    if not args.no_shapes:
+        out["shapes"] = shape_table(torch, msd, dev, stream)
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(step.bytes)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -56,10 +56,18 @@ int msd_shutdown(void);
 int msd_status(void *stream);
 
 /*
- * Tuning knob: msd_groupnorm splits each (sample, group) over enough
- * workgroups to reach about this many per launch (default 512).
+ * Tuning / test knob: forces how msd_groupnorm cuts each (sample, group) into
+ * workgroups.  split = workgroups per group (power of two <= 64, 0 = automatic;
+ * a value below what fits in registers is raised), threads = workgroup size
+ * (multiple of 64 <= 1024, 0 = automatic).  Process-wide.
  */
-int msd_set_groupnorm_target_blocks(int blocks);
+int msd_set_groupnorm_plan(int split, int threads);
+
+/*
+ * Tuning / test knob: bytes each lane of msd_layernorm moves per load (8 or 16;
+ * 0 = automatic).  Process-wide.
+ */
+int msd_set_layernorm_chunk(int bytes);
 
 /*
  * GroupNorm over NCHW, optionally followed by SiLU, in one launch.

@@ -36,9 +36,22 @@ def _run(cmd):
     return out
 
 
+HIP_SOURCES = ["api.hip", "groupnorm.hip", "layernorm.hip", "stream_ops.hip"]
+
+
 def build_hip():
-    src = os.path.join(CSRC, "msd_kernels.hip")
-    _run([HIPCC] + DEVICE_FLAGS + ["-shared", "-o", LIB_HIP, src])
+    """Compiles each translation unit to an object (in parallel) and links libmsd_hip.so."""
+    from concurrent.futures import ThreadPoolExecutor
+    objs = [os.path.join(CSRC, s.replace(".hip", ".o")) for s in HIP_SOURCES]
+
+    def compile_one(pair):
+        src, obj = pair
+        return _run([HIPCC] + DEVICE_FLAGS + ["-c", "-o", obj, os.path.join(CSRC, src)])
+
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        list(pool.map(compile_one, zip(HIP_SOURCES, objs)))
+    _run([HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-Wno-unused-command-line-argument",
+          "-o", LIB_HIP] + objs)
     return LIB_HIP
 
 

@@ -1,0 +1,208 @@
+// C ABI of libmsd_hip.so (declared in include/msd_hip.h): argument checks, dtype
+// dispatch and the per-(device, stream) GroupNorm scratch.
+#include <cmath>
+#include <mutex>
+#include <unordered_map>
+
+#include <hip/hip_fp16.h>
+
+#include "msd_internal.h"
+
+namespace msd {
+namespace {
+
+struct ScratchKey {
+    int device;
+    hipStream_t stream;
+    bool operator==(const ScratchKey &o) const { return device == o.device && stream == o.stream; }
+};
+struct ScratchKeyHash {
+    size_t operator()(const ScratchKey &k) const {
+        return std::hash<void *>()((void *)k.stream) ^ (std::hash<int>()(k.device) * 0x9E3779B1u);
+    }
+};
+
+std::mutex g_scratch_mutex;
+std::unordered_map<ScratchKey, GnScratch, ScratchKeyHash> g_scratch;
+
+constexpr size_t kSlotBytes = sizeof(unsigned long long) * kGnMaxUnits * kGnMaxSplit;
+constexpr size_t kWordBytes = sizeof(uint32_t) * kGnMaxUnits;
+constexpr size_t kScratchBytes = 2 * kSlotBytes + 2 * kWordBytes + 256;
+
+}  // namespace
+
+// Scratch is private to a (device, stream) pair: launches on one stream are ordered, so a
+// unit's slots are never shared by two launches in flight.
+hipError_t get_scratch(hipStream_t stream, GnScratch *out) {
+    int device = 0;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess) return err;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    const ScratchKey key{device, stream};
+    auto it = g_scratch.find(key);
+    if (it != g_scratch.end()) {
+        *out = it->second;
+        return hipSuccess;
+    }
+    char *base = nullptr;
+    err = hipMalloc(reinterpret_cast<void **>(&base), kScratchBytes);
+    if (err != hipSuccess) return err;
+    err = hipMemset(base, 0, kScratchBytes);  // tags, epochs and counters start at zero
+    if (err != hipSuccess) {
+        (void)hipFree(base);
+        return err;
+    }
+    GnScratch s;
+    s.slot_mean = reinterpret_cast<unsigned long long *>(base);
+    s.slot_m2 = reinterpret_cast<unsigned long long *>(base + kSlotBytes);
+    s.epoch = reinterpret_cast<uint32_t *>(base + 2 * kSlotBytes);
+    s.done = reinterpret_cast<uint32_t *>(base + 2 * kSlotBytes + kWordBytes);
+    s.status = reinterpret_cast<uint32_t *>(base + 2 * kSlotBytes + 2 * kWordBytes);
+    g_scratch.emplace(key, s);
+    *out = s;
+    return hipSuccess;
+}
+
+}  // namespace msd
+
+using namespace msd;
+
+extern "C" {
+
+int msd_version(void) { return 100; }
+
+const char *msd_error_string(int code) {
+    if (code == MSD_OK) return "ok";
+    if (code == MSD_ERR_INVALID_VALUE) return "invalid value (shape, pointer or dtype rejected)";
+    return hipGetErrorString(static_cast<hipError_t>(code));
+}
+
+int msd_init(void *stream) {
+    GnScratch sc;
+    return (int)get_scratch(static_cast<hipStream_t>(stream), &sc);
+}
+
+int msd_shutdown(void) {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    int rc = MSD_OK;
+    int current = 0;
+    (void)hipGetDevice(&current);
+    for (auto &kv : g_scratch) {
+        (void)hipSetDevice(kv.first.device);
+        const hipError_t err = hipFree(kv.second.slot_mean);
+        if (err != hipSuccess) rc = (int)err;
+    }
+    g_scratch.clear();
+    (void)hipSetDevice(current);
+    return rc;
+}
+
+int msd_status(void *stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipError_t err = hipStreamSynchronize(s);
+    if (err != hipSuccess) return (int)err;
+    int device = 0;
+    err = hipGetDevice(&device);
+    if (err != hipSuccess) return (int)err;
+    GnScratch sc;
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        auto it = g_scratch.find(ScratchKey{device, s});
+        if (it == g_scratch.end()) return MSD_OK;
+        sc = it->second;
+    }
+    uint32_t flags = 0;
+    err = hipMemcpy(&flags, sc.status, sizeof(flags), hipMemcpyDeviceToHost);
+    if (err != hipSuccess) return (int)err;
+    return flags ? (int)hipErrorLaunchFailure : MSD_OK;
+}
+
+int msd_set_groupnorm_plan(int split, int threads) {
+    if (split < 0 || threads < 0) return MSD_ERR_INVALID_VALUE;
+    if (split > 0 && ((split & (split - 1)) != 0 || split > (int)kGnMaxSplit)) return MSD_ERR_INVALID_VALUE;
+    if (threads > 0 && (threads % 64 != 0 || threads > 1024)) return MSD_ERR_INVALID_VALUE;
+    g_gn_plan_override.split = split;
+    g_gn_plan_override.threads = threads;
+    return MSD_OK;
+}
+
+int msd_set_layernorm_chunk(int bytes) {
+    if (bytes != 0 && bytes != 8 && bytes != 16) return MSD_ERR_INVALID_VALUE;
+    g_ln_chunk_override = bytes;
+    return MSD_OK;
+}
+
+int msd_groupnorm(const void *x, void *y, const float *gamma, const float *beta, size_t batch,
+                  size_t channels, size_t hw, size_t groups, float eps, int fuse_silu, int dtype,
+                  void *stream) {
+    if (groups == 0 || channels == 0 || channels % groups != 0) return MSD_ERR_INVALID_VALUE;
+    if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
+    if (batch * hw != 0 && (!x || !y || !gamma || !beta)) return MSD_ERR_INVALID_VALUE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == MSD_DTYPE_F32)
+        return gn_dispatch<float>(x, y, gamma, beta, batch, channels, hw, groups, eps,
+                                  fuse_silu != 0, s);
+    return gn_dispatch<__half>(x, y, gamma, beta, batch, channels, hw, groups, eps, fuse_silu != 0,
+                               s);
+}
+
+int msd_layernorm(const void *x, void *y, const float *gamma, const float *beta, size_t rows,
+                  size_t dim, float eps, int dtype, void *stream) {
+    if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
+    if (rows * dim != 0 && (!x || !y || !gamma || !beta)) return MSD_ERR_INVALID_VALUE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == MSD_DTYPE_F32) return ln_dispatch<float>(x, y, gamma, beta, rows, dim, eps, s);
+    return ln_dispatch<__half>(x, y, gamma, beta, rows, dim, eps, s);
+}
+
+int msd_geglu(const void *proj, void *out, size_t rows, size_t inner, int dtype, void *stream) {
+    if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
+    if (rows * inner != 0 && (!proj || !out)) return MSD_ERR_INVALID_VALUE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == MSD_DTYPE_F32) return geglu_dispatch<float>(proj, out, rows, inner, s);
+    return geglu_dispatch<__half>(proj, out, rows, inner, s);
+}
+
+static int act_entry(Act op, const void *x, void *y, size_t n, int dtype, void *stream) {
+    if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
+    if (n != 0 && (!x || !y)) return MSD_ERR_INVALID_VALUE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == MSD_DTYPE_F32) return act_dispatch<float>(op, x, y, n, s);
+    return act_dispatch<__half>(op, x, y, n, s);
+}
+
+int msd_silu(const void *x, void *y, size_t n, int dtype, void *stream) {
+    return act_entry(Act::Silu, x, y, n, dtype, stream);
+}
+int msd_gelu(const void *x, void *y, size_t n, int dtype, void *stream) {
+    return act_entry(Act::Gelu, x, y, n, dtype, stream);
+}
+int msd_quick_gelu(const void *x, void *y, size_t n, int dtype, void *stream) {
+    return act_entry(Act::QuickGelu, x, y, n, dtype, stream);
+}
+
+int msd_timestep_embedding(const int64_t *timesteps, void *out, size_t batch, size_t dim,
+                           float max_period, int dtype, void *stream) {
+    if (dim % 2 != 0 || !(max_period > 0.0f)) return MSD_ERR_INVALID_VALUE;
+    if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
+    if (batch * dim == 0) return MSD_OK;
+    if (!timesteps || !out || batch * dim > 0x7FFFFFFFull) return MSD_ERR_INVALID_VALUE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == MSD_DTYPE_F32)
+        return temb_dispatch<float>(timesteps, out, batch, dim, max_period, s);
+    return temb_dispatch<__half>(timesteps, out, batch, dim, max_period, s);
+}
+
+int msd_ddim_timesteps(int ddim_num_steps, int *out, int cap) {
+    const int ddpm_steps = 1000;
+    if (ddim_num_steps < 1 || ddim_num_steps > ddpm_steps) return -1;
+    const int stride = ddpm_steps / ddim_num_steps;
+    int count = 0;
+    for (int t = 1; t <= ddpm_steps; t += stride) {
+        if (out && count < cap) out[count] = t;
+        count++;
+    }
+    return count;
+}
+
+}  // extern "C"

@@ -1,0 +1,459 @@
+// GroupNorm (+ SiLU) for gfx950.
+//
+// A unit is one (sample, group): ch_per_group * hw contiguous elements of an
+// NCHW tensor.  A unit is cut into `split` slices, one workgroup per slice; the
+// slice stays in registers as packed 16-byte vectors for the whole kernel, so
+// the tensor is read from HBM once and written once.
+//
+//   1. every lane issues all its loads (K vectors) before the first use;
+//   2. slice mean, then slice M2 = sum (x - slice mean)^2, both from registers
+//      (DPP wavefront reduction, one LDS slot per wavefront);
+//   3. split > 1: slices publish (mean, M2) as two tagged 64-bit words, poll
+//      their siblings' words, and merge with Chan's formula.  The tag is the
+//      unit's launch count, read at kernel start; the last slice to finish
+//      advances it, so nothing is reset between launches and a replayed graph
+//      works.  All traffic is relaxed agent-scope atomics: no cache flushes.
+//   4. y = fma(x - mean, rstd * gamma[c], beta[c]), optional SiLU, packed store.
+//
+// Workgroups of one unit have adjacent block ids, so every workgroup a waiter
+// depends on is dispatched no later than the waiter; waits are also bounded.
+#include "msd_device.h"
+#include "msd_internal.h"
+
+namespace msd {
+
+GnPlanOverride g_gn_plan_override = {0, 0};
+
+namespace {
+
+constexpr int kGnMaxThreads = 1024;
+constexpr int kGnMaxK = 16;
+constexpr uint32_t kGnSpinLimit = 1u << 22;
+constexpr int kGenericThreads = 256;
+
+struct GnParams {
+    uint32_t vec_per_unit;   // 16-byte vectors per unit
+    uint32_t vec_per_slice;  // vectors per workgroup (the last slice may be shorter)
+    uint32_t split;          // workgroups per unit, power of two <= kGnMaxSplit
+    uint32_t split_shift;    // log2(split)
+    uint32_t groups;
+    uint32_t ch_per_group;
+    FastDiv hw_vec;          // vectors per channel
+    float eps;
+    float inv_count;         // 1 / elements per unit
+};
+
+// Sum over the workgroup (blockDim.x / 64 wavefronts); one barrier.
+__device__ __forceinline__ float block_sum_rt(float v, float *slots) {
+    const float w = wave_sum(v);
+    const uint32_t nw = blockDim.x / kWave;
+    if ((threadIdx.x & (kWave - 1)) == 0) slots[threadIdx.x / kWave] = w;
+    __syncthreads();
+    float t = 0.0f;
+    for (uint32_t i = 0; i < nw; i++) t += slots[i];
+    return t;
+}
+
+__device__ __forceinline__ unsigned long long tagged(uint32_t tag, float v) {
+    return ((unsigned long long)tag << 32) | (unsigned long long)__float_as_uint(v);
+}
+
+// FULL: every lane owns exactly K vectors (no masking anywhere).
+template <typename T, int K, bool SILU, bool FULL>
+__device__ __forceinline__ void gn_body(const T *x, T *y, const float *__restrict__ gamma,
+                                        const float *__restrict__ beta, const GnScratch &scratch,
+                                        const GnParams &p, uint32_t unit, uint32_t slice,
+                                        uint32_t v_begin, uint32_t v_end, float *red_a,
+                                        float *red_b, float *stats) {
+    constexpr int EPV = Store<T>::EPV;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t nt = blockDim.x;
+    const u32x4 *xin = reinterpret_cast<const u32x4 *>(x) + (size_t)unit * p.vec_per_unit;
+    u32x4 *yout = reinterpret_cast<u32x4 *>(y) + (size_t)unit * p.vec_per_unit;
+
+    // launch count of this unit: the tag of this launch's exchange (latency hidden by the loads)
+    uint32_t epoch = 0;
+    if (p.split > 1 && tid == 0)
+        epoch = __hip_atomic_load(scratch.epoch + unit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+    // ---- the slice goes into registers.  Lanes past the end of a ragged slice re-read its
+    // last vector (a valid address) and are masked later: no load sits behind a branch.
+    u32x4 raw[K];
+    uint32_t vidx[K];
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        const uint32_t v = v_begin + k * nt + tid;
+        vidx[k] = FULL ? v : min(v, v_end - 1);
+        raw[k] = load_stream(xin + vidx[k]);
+    }
+    // per-vector channel affine: fetched up front while the data is in flight when the
+    // registers allow it, otherwise just before use
+    constexpr bool kPrefetchAffine = K <= 6;
+    const uint32_t ch0 = (unit % p.groups) * p.ch_per_group;
+    float ga[kPrefetchAffine ? K : 1], be[kPrefetchAffine ? K : 1];
+    if (kPrefetchAffine) {
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            const uint32_t c = ch0 + fast_div(vidx[k], p.hw_vec);
+            ga[kPrefetchAffine ? k : 0] = gamma[c];
+            be[kPrefetchAffine ? k : 0] = beta[c];
+        }
+    }
+
+    // ---- slice mean
+    float s = 0.0f;
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        float f[EPV];
+        Store<T>::unpack(raw[k], f);
+        float sk = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EPV; e++) sk += f[e];
+        if (!FULL) sk = (v_begin + k * nt + tid < v_end) ? sk : 0.0f;
+        s += sk;
+    }
+    const float slice_count = (float)((v_end - v_begin) * EPV);
+    const float slice_mean = block_sum_rt(s, red_a) / slice_count;
+    if (sizeof(T) == 2) {
+#pragma unroll
+        for (int k = 0; k < K; k++) forget(raw[k]);
+    }
+
+    // ---- slice M2
+    float q = 0.0f;
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        float f[EPV];
+        Store<T>::unpack(raw[k], f);
+        float qk = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EPV; e++) {
+            const float d = f[e] - slice_mean;
+            qk = fmaf(d, d, qk);
+        }
+        if (!FULL) qk = (v_begin + k * nt + tid < v_end) ? qk : 0.0f;
+        q += qk;
+    }
+    const float slice_m2 = block_sum_rt(q, red_b);
+    if (sizeof(T) == 2) {
+#pragma unroll
+        for (int k = 0; k < K; k++) forget(raw[k]);
+    }
+
+    float mean, rstd;
+    if (p.split == 1) {
+        mean = slice_mean;
+        rstd = __builtin_amdgcn_rsqf(slice_m2 * p.inv_count + p.eps);
+    } else {
+        unsigned long long *slot_mean = scratch.slot_mean + (size_t)unit * kGnMaxSplit;
+        unsigned long long *slot_m2 = scratch.slot_m2 + (size_t)unit * kGnMaxSplit;
+        if (tid < kWave) {  // wavefront 0 owns the exchange; lane 0 holds the epoch
+            const uint32_t tag =
+                (uint32_t)__builtin_amdgcn_readfirstlane((int)epoch) + 1u;
+            if (tid == 0) {
+                __hip_atomic_store(slot_mean + slice, tagged(tag, slice_mean), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(slot_m2 + slice, tagged(tag, slice_m2), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            }
+            // lane l waits for slice l
+            float m_l = 0.0f, q_l = 0.0f, n_l = 0.0f;
+            if (tid < p.split) {
+                unsigned long long wm, wq;
+                uint32_t polls = 0;
+                bool ok;
+                do {
+                    wm = __hip_atomic_load(slot_mean + tid, __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+                    wq = __hip_atomic_load(slot_m2 + tid, __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+                    ok = (uint32_t)(wm >> 32) == tag && (uint32_t)(wq >> 32) == tag;
+                    if (!ok) __builtin_amdgcn_s_sleep(1);
+                } while (!ok && ++polls < kGnSpinLimit);
+                if (!ok)
+                    __hip_atomic_fetch_or(scratch.status, 1u, __ATOMIC_RELAXED,
+                                          __HIP_MEMORY_SCOPE_AGENT);
+                m_l = __uint_as_float((uint32_t)wm);
+                q_l = __uint_as_float((uint32_t)wq);
+                const uint32_t b = tid * p.vec_per_slice;
+                const uint32_t e = min(p.vec_per_unit, b + p.vec_per_slice);
+                n_l = (float)((e - b) * EPV);
+            }
+            // Chan: mean = sum n_l mean_l / n ; M2 = sum M2_l + sum n_l (mean_l - mean)^2
+            const float total_mean = wave_sum(m_l * n_l) * p.inv_count;
+            const float dm = m_l - total_mean;
+            const float m2 = wave_sum(fmaf(n_l * dm, dm, q_l));
+            if (tid == 0) {
+                stats[0] = total_mean;
+                stats[1] = __builtin_amdgcn_rsqf(m2 * p.inv_count + p.eps);
+                // this slice has consumed its siblings' words; the last one closes the launch
+                const uint32_t old = __hip_atomic_fetch_add(scratch.done + unit, 1u, __ATOMIC_RELAXED,
+                                                            __HIP_MEMORY_SCOPE_AGENT);
+                if (old == p.split - 1) {
+                    __hip_atomic_store(scratch.done + unit, 0u, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(scratch.epoch + unit, tag, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+        }
+        __syncthreads();
+        mean = stats[0];
+        rstd = stats[1];
+    }
+
+    // ---- normalise from registers, per-channel affine, optional SiLU
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        float g_k, b_k;
+        if (kPrefetchAffine) {
+            g_k = ga[kPrefetchAffine ? k : 0];
+            b_k = be[kPrefetchAffine ? k : 0];
+        } else {
+            const uint32_t c = ch0 + fast_div(vidx[k], p.hw_vec);
+            g_k = gamma[c];
+            b_k = beta[c];
+        }
+        const float a = rstd * g_k;
+        float f[EPV];
+        Store<T>::unpack(raw[k], f);
+#pragma unroll
+        for (int e = 0; e < EPV; e++) {
+            const float t = fmaf(f[e] - mean, a, b_k);
+            f[e] = SILU ? silu_f(t) : t;
+        }
+        const u32x4 packed = Store<T>::pack(f);
+        if (FULL || v_begin + k * nt + tid < v_end) store_stream(yout + vidx[k], packed);
+    }
+}
+
+template <typename T, int K, bool SILU>
+__global__ __launch_bounds__(kGnMaxThreads) void gn_slice_kernel(
+    const T *x, T *y, const float *__restrict__ gamma, const float *__restrict__ beta,
+    GnScratch scratch, GnParams p) {
+    __shared__ float red_a[kGnMaxThreads / kWave];
+    __shared__ float red_b[kGnMaxThreads / kWave];
+    __shared__ float stats[2];
+    const uint32_t unit = blockIdx.x >> p.split_shift;
+    const uint32_t slice = blockIdx.x & (p.split - 1);
+    const uint32_t v_begin = slice * p.vec_per_slice;
+    const uint32_t v_end = min(p.vec_per_unit, v_begin + p.vec_per_slice);
+    if (v_end - v_begin == K * blockDim.x)  // uniform over the workgroup
+        gn_body<T, K, SILU, true>(x, y, gamma, beta, scratch, p, unit, slice, v_begin, v_end, red_a,
+                                  red_b, stats);
+    else
+        gn_body<T, K, SILU, false>(x, y, gamma, beta, scratch, p, unit, slice, v_begin, v_end,
+                                   red_a, red_b, stats);
+}
+
+// Any shape or alignment: one workgroup per unit, three passes over global memory with
+// scalar accesses (the second and third pass hit in cache for UNet-sized units).
+template <typename T, bool SILU>
+__global__ __launch_bounds__(kGenericThreads) void gn_generic_kernel(
+    const T *x, T *y, const float *__restrict__ gamma, const float *__restrict__ beta,
+    uint32_t unit_size, uint32_t hw, uint32_t groups, uint32_t ch_per_group, float eps) {
+    __shared__ float red_a[kGenericThreads / kWave];
+    __shared__ float red_b[kGenericThreads / kWave];
+    const uint32_t unit = blockIdx.x;
+    const T *xin = x + (size_t)unit * unit_size;
+    T *yout = y + (size_t)unit * unit_size;
+    float s = 0.0f;
+    for (uint32_t i = threadIdx.x; i < unit_size; i += kGenericThreads) s += Store<T>::load1(xin + i);
+    const float mean = block_sum_rt(s, red_a) / (float)unit_size;
+    float q = 0.0f;
+    for (uint32_t i = threadIdx.x; i < unit_size; i += kGenericThreads) {
+        const float d = Store<T>::load1(xin + i) - mean;
+        q = fmaf(d, d, q);
+    }
+    const float rstd = 1.0f / sqrtf(block_sum_rt(q, red_b) / (float)unit_size + eps);
+    const uint32_t ch0 = (unit % groups) * ch_per_group;
+    for (uint32_t i = threadIdx.x; i < unit_size; i += kGenericThreads) {
+        const uint32_t c = ch0 + i / hw;
+        const float t = fmaf(Store<T>::load1(xin + i) - mean, rstd * gamma[c], beta[c]);
+        Store<T>::store1(yout + i, SILU ? silu_f(t) : t);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Host: launch plan
+// ---------------------------------------------------------------------------
+FastDiv make_fast_div(uint32_t d) {
+    FastDiv fd{0u, 0u, d};
+    if (d <= 1) return fd;
+    uint32_t L = 0;
+    while ((1ull << L) < d) L++;
+    fd.mul = (uint32_t)(((1ull << (31 + L)) + d - 1) / d);
+    fd.shift = L - 1;
+    return fd;
+}
+
+const int kKValues[] = {1, 2, 3, 4, 5, 6, 8, 10, 12, 16};
+
+inline int round_up_k(uint32_t k) {
+    for (int v : kKValues)
+        if ((uint32_t)v >= k) return v;
+    return 0;
+}
+
+struct GnPlan {
+    uint32_t split;
+    uint32_t threads;
+    int k;  // 0 = does not fit
+};
+
+// Threads and K for a slice of `vecs` vectors.  Measured on MI355X, workgroups of about
+// 512 lanes finish soonest (enough wavefronts to hide latency, short reduction tail), so
+// among the widths (multiples of 64 in [256, 1024]) that divide the slice into one of the
+// compiled K values the one nearest 512 wins; without an exact fit the tail is masked.
+GnPlan plan_slice(uint32_t vecs, uint32_t split, uint32_t force_threads, uint32_t max_k) {
+    GnPlan pl{split, 0, 0};
+    if (force_threads) {
+        pl.threads = force_threads;
+        pl.k = round_up_k((vecs + force_threads - 1) / force_threads);
+        if ((uint32_t)pl.k > max_k) pl.k = 0;
+        return pl;
+    }
+    uint32_t best_nt = 0, best_dist = ~0u;
+    for (uint32_t nt = 256; nt <= (uint32_t)kGnMaxThreads; nt += kWave) {
+        if (vecs % nt) continue;
+        const uint32_t k = vecs / nt;
+        if (k > max_k || round_up_k(k) != (int)k) continue;
+        const uint32_t dist = nt > 512 ? nt - 512 : 512 - nt;
+        if (dist < best_dist) {
+            best_dist = dist;
+            best_nt = nt;
+        }
+    }
+    if (best_nt) {
+        pl.threads = best_nt;
+        pl.k = (int)(vecs / best_nt);
+        return pl;
+    }
+    if (vecs > 512u * max_k)
+        pl.threads = kGnMaxThreads;
+    else if (vecs >= 512)
+        pl.threads = 512;
+    else
+        pl.threads = ((vecs + kWave - 1) / kWave) * kWave;
+    pl.k = round_up_k((vecs + pl.threads - 1) / pl.threads);
+    if ((uint32_t)pl.k > max_k) pl.k = 0;
+    return pl;
+}
+
+template <typename T, int K>
+void gn_launch_k(bool silu, uint32_t blocks, uint32_t threads, hipStream_t stream, const T *x, T *y,
+                 const float *gamma, const float *beta, const GnScratch &sc, const GnParams &p) {
+    if (silu)
+        hipLaunchKernelGGL((gn_slice_kernel<T, K, true>), dim3(blocks), dim3(threads), 0, stream, x,
+                           y, gamma, beta, sc, p);
+    else
+        hipLaunchKernelGGL((gn_slice_kernel<T, K, false>), dim3(blocks), dim3(threads), 0, stream,
+                           x, y, gamma, beta, sc, p);
+}
+
+template <typename T>
+int gn_generic(bool silu, const T *x, T *y, const float *gamma, const float *beta, size_t units,
+               size_t unit_size, size_t hw, size_t groups, size_t cpg, float eps,
+               hipStream_t stream) {
+    hipLaunchKernelGGL((silu ? gn_generic_kernel<T, true> : gn_generic_kernel<T, false>),
+                       dim3((uint32_t)units), dim3(kGenericThreads), 0, stream, x, y, gamma, beta,
+                       (uint32_t)unit_size, (uint32_t)hw, (uint32_t)groups, (uint32_t)cpg, eps);
+    return launch_status();
+}
+
+}  // namespace
+
+template <typename T>
+int gn_dispatch(const void *xv, void *yv, const float *gamma, const float *beta, size_t batch,
+                size_t channels, size_t hw, size_t groups, float eps, bool silu,
+                hipStream_t stream) {
+    constexpr int EPV = Store<T>::EPV;
+    const T *x = static_cast<const T *>(xv);
+    T *y = static_cast<T *>(yv);
+    const size_t cpg = channels / groups;
+    const size_t unit_size = cpg * hw;
+    const size_t units = batch * groups;
+    if (units == 0 || unit_size == 0) return MSD_OK;
+    if (units > 0x7FFFFFFFull || unit_size > 0x7FFFFFFFull) return MSD_ERR_INVALID_VALUE;
+    if (!(aligned16(x) && aligned16(y) && hw % EPV == 0))
+        return gn_generic<T>(silu, x, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
+
+    const size_t vec_per_unit = unit_size / EPV;
+    // vectors per lane that stay in registers without spilling under the 1024-lane bound
+    constexpr uint32_t kMaxK = sizeof(T) == 4 ? 10 : kGnMaxK;
+    const size_t slice_cap = (size_t)kGnMaxThreads * kMaxK;  // vectors one workgroup can hold
+    // smallest power-of-two split whose slices fit in registers
+    uint32_t split = 1;
+    while ((size_t)split * slice_cap < vec_per_unit && split <= kGnMaxSplit) split *= 2;
+    const bool can_split = units <= kGnMaxUnits;
+    if (split > kGnMaxSplit || (split > 1 && !can_split))
+        return gn_generic<T>(silu, x, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
+    if (g_gn_plan_override.split > 0) {
+        uint32_t forced = (uint32_t)g_gn_plan_override.split;
+        if (forced > split && can_split && (forced & (forced - 1)) == 0 && forced <= kGnMaxSplit &&
+            vec_per_unit >= (size_t)forced * kWave)
+            split = forced;
+    } else if (can_split) {
+        // A workgroup's time grows with its slice (about 0.13 us per 1024 elements on MI355X,
+        // it is latency- and ALU-bound, not bandwidth-bound) while the exchange between the
+        // slices of a unit costs 1.3 - 2.5 us, so units up to 24 Ki elements stay whole and
+        // larger ones are cut in four; eight when that still leaves most of the chip idle.
+        uint32_t want = 1;
+        if (unit_size > 24576) {
+            want = 4;
+            if (units * 4 < 192 && unit_size >= 65536) want = 8;
+        }
+        while (units * want < 16 && want < kGnMaxSplit) want *= 2;  // very few units
+        while (split < want && vec_per_unit >= (size_t)2 * split * 256) split *= 2;
+    }
+
+    GnParams p;
+    p.vec_per_unit = (uint32_t)vec_per_unit;
+    p.vec_per_slice = (uint32_t)((vec_per_unit + split - 1) / split);
+    p.split = split;
+    p.split_shift = (uint32_t)__builtin_ctz(split);
+    p.groups = (uint32_t)groups;
+    p.ch_per_group = (uint32_t)cpg;
+    p.hw_vec = make_fast_div((uint32_t)(hw / EPV));
+    p.eps = eps;
+    p.inv_count = 1.0f / (float)unit_size;
+    // every slice must own at least one vector (ceil division can starve the last ones)
+    if ((size_t)p.vec_per_slice * (split - 1) >= vec_per_unit)
+        return gn_generic<T>(silu, x, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
+
+    uint32_t force_threads = 0;
+    if (g_gn_plan_override.threads >= kWave && g_gn_plan_override.threads <= kGnMaxThreads &&
+        g_gn_plan_override.threads % kWave == 0 &&
+        (size_t)g_gn_plan_override.threads * kMaxK >= p.vec_per_slice)
+        force_threads = (uint32_t)g_gn_plan_override.threads;
+    const GnPlan pl = plan_slice(p.vec_per_slice, split, force_threads, kMaxK);
+    if (pl.k == 0)
+        return gn_generic<T>(silu, x, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
+
+    GnScratch sc{nullptr, nullptr, nullptr, nullptr, nullptr};
+    if (split > 1) {
+        const hipError_t err = get_scratch(stream, &sc);
+        if (err != hipSuccess) return (int)err;
+    }
+    const uint32_t blocks = (uint32_t)(units * split);
+    switch (pl.k) {
+        case 1: gn_launch_k<T, 1>(silu, blocks, pl.threads, stream, x, y, gamma, beta, sc, p); break;
+        case 2: gn_launch_k<T, 2>(silu, blocks, pl.threads, stream, x, y, gamma, beta, sc, p); break;
+        case 3: gn_launch_k<T, 3>(silu, blocks, pl.threads, stream, x, y, gamma, beta, sc, p); break;
+        case 4: gn_launch_k<T, 4>(silu, blocks, pl.threads, stream, x, y, gamma, beta, sc, p); break;
+        case 5: gn_launch_k<T, 5>(silu, blocks, pl.threads, stream, x, y, gamma, beta, sc, p); break;
+        case 6: gn_launch_k<T, 6>(silu, blocks, pl.threads, stream, x, y, gamma, beta, sc, p); break;
+        case 8: gn_launch_k<T, 8>(silu, blocks, pl.threads, stream, x, y, gamma, beta, sc, p); break;
+        case 10: gn_launch_k<T, 10>(silu, blocks, pl.threads, stream, x, y, gamma, beta, sc, p); break;
+        case 12: gn_launch_k<T, 12>(silu, blocks, pl.threads, stream, x, y, gamma, beta, sc, p); break;
+        default: gn_launch_k<T, 16>(silu, blocks, pl.threads, stream, x, y, gamma, beta, sc, p); break;
+    }
+    return launch_status();
+}
+
+template int gn_dispatch<float>(const void *, void *, const float *, const float *, size_t, size_t,
+                                size_t, size_t, float, bool, hipStream_t);
+template int gn_dispatch<__half>(const void *, void *, const float *, const float *, size_t, size_t,
+                                 size_t, size_t, float, bool, hipStream_t);
+
+}  // namespace msd

@@ -1,0 +1,256 @@
+// LayerNorm for gfx950: a row is owned by a team of TL adjacent lanes of one
+// wavefront (TL = 4..64), VPL 16-byte vectors per lane, so a wavefront covers
+// 64/TL consecutive rows and every load instruction fetches whole 128-byte lines.
+// Mean and M2 are computed from registers in two passes (exact centred variance),
+// reduced across the team with DPP; gamma / beta are fetched while the row data is
+// in flight.  One HBM read and one HBM write per element.
+#include "msd_device.h"
+#include "msd_internal.h"
+
+namespace msd {
+namespace {
+
+constexpr int kLnThreads = 256;
+
+// NW dwords (8 or 16 bytes) of T, moved with one instruction.
+template <int NW>
+struct Words;
+template <>
+struct Words<4> {
+    typedef u32x4 type;
+};
+template <>
+struct Words<2> {
+    typedef uint32_t type __attribute__((ext_vector_type(2)));
+};
+
+template <typename T, int NW>
+struct Chunk {
+    static constexpr int N = NW * 4 / (int)sizeof(T);  // elements per chunk
+    typedef typename Words<NW>::type vec_t;
+    static __device__ __forceinline__ void unpack(const vec_t &v, float *f) {
+        if (sizeof(T) == 4) {
+#pragma unroll
+            for (int i = 0; i < NW; i++) f[i] = __uint_as_float(v[i]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < NW; i++) {
+                const uint32_t w = v[i];
+                const float2 t = __half22float2(*reinterpret_cast<const __half2 *>(&w));
+                f[2 * i] = t.x;
+                f[2 * i + 1] = t.y;
+            }
+        }
+    }
+    static __device__ __forceinline__ vec_t pack(const float *f) {
+        vec_t v;
+        if (sizeof(T) == 4) {
+#pragma unroll
+            for (int i = 0; i < NW; i++) v[i] = __float_as_uint(f[i]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < NW; i++) {
+                const __half2 h = __floats2half2_rn(f[2 * i], f[2 * i + 1]);
+                v[i] = *reinterpret_cast<const uint32_t *>(&h);
+            }
+        }
+        return v;
+    }
+};
+
+// A row of VPL*TL chunks (NW dwords each) is owned by TL adjacent lanes; a wavefront
+// covers 64/TL consecutive rows.  Lane (team, j) holds chunks j, j+TL, ... of its row and
+// the gamma / beta of the same columns, all requested before the first use.
+template <typename T, int NW, int VPL, int TL>
+__global__ __launch_bounds__(kLnThreads) void ln_team_kernel(
+    const T *x, T *y, const float *__restrict__ gamma, const float *__restrict__ beta,
+    uint32_t rows, float eps, float inv_dim) {
+    typedef Chunk<T, NW> C;
+    typedef typename C::vec_t vec_t;
+    constexpr int N = C::N;
+    constexpr int RPW = kWave / TL;  // rows per wavefront
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = blockIdx.x * (kLnThreads / kWave) + threadIdx.x / kWave;
+    const uint32_t row = wave * RPW + lane / TL;
+    const uint32_t j = lane % TL;
+    const bool live = row < rows;
+    // lanes past the last row re-read it (valid address, no branch around the loads)
+    const size_t row_chunk = (size_t)min(row, rows - 1) * (VPL * TL);
+    const vec_t *xin = reinterpret_cast<const vec_t *>(x) + row_chunk;
+    vec_t *yout = reinterpret_cast<vec_t *>(y) + row_chunk;
+
+    vec_t raw[VPL];
+#pragma unroll
+    for (int k = 0; k < VPL; k++) raw[k] = __builtin_nontemporal_load(xin + k * TL + j);
+    float g[VPL][N], b[VPL][N];
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+        const uint32_t col = (k * TL + j) * N;
+#pragma unroll
+        for (int e = 0; e < N; e += (N >= 4 ? 4 : 2)) {
+            if (N >= 4) {
+                const f32x4 gv = *reinterpret_cast<const f32x4 *>(gamma + col + e);
+                const f32x4 bv = *reinterpret_cast<const f32x4 *>(beta + col + e);
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    g[k][e + i] = gv[i];
+                    b[k][e + i] = bv[i];
+                }
+            } else {
+                const float2 gv = *reinterpret_cast<const float2 *>(gamma + col + e);
+                const float2 bv = *reinterpret_cast<const float2 *>(beta + col + e);
+                g[k][e] = gv.x;
+                g[k][e + 1] = gv.y;
+                b[k][e] = bv.x;
+                b[k][e + 1] = bv.y;
+            }
+        }
+    }
+    float f[VPL][N];
+    float s = 0.0f;
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+        C::unpack(raw[k], f[k]);
+#pragma unroll
+        for (int e = 0; e < N; e++) s += f[k][e];
+    }
+    const float mean = team_sum<TL>(s) * inv_dim;
+    float q = 0.0f;
+#pragma unroll
+    for (int k = 0; k < VPL; k++)
+#pragma unroll
+        for (int e = 0; e < N; e++) {
+            f[k][e] -= mean;
+            q = fmaf(f[k][e], f[k][e], q);
+        }
+    const float rstd = __builtin_amdgcn_rsqf(team_sum<TL>(q) * inv_dim + eps);
+    if (!live) return;
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+        float o[N];
+#pragma unroll
+        for (int e = 0; e < N; e++) o[e] = fmaf(f[k][e] * rstd, g[k][e], b[k][e]);
+        __builtin_nontemporal_store(C::pack(o), yout + k * TL + j);
+    }
+}
+
+// Any dim: one wavefront per row, scalar accesses, three passes.
+template <typename T>
+__global__ __launch_bounds__(kLnThreads) void ln_generic_kernel(
+    const T *x, T *y, const float *__restrict__ gamma,
+    const float *__restrict__ beta, uint32_t rows, uint32_t dim, float eps) {
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t row = blockIdx.x * (kLnThreads / kWave) + threadIdx.x / kWave;
+    if (row >= rows) return;  // whole wavefront leaves together
+    const T *xin = x + (size_t)row * dim;
+    T *yout = y + (size_t)row * dim;
+    float s = 0.0f;
+    for (uint32_t i = lane; i < dim; i += kWave) s += Store<T>::load1(xin + i);
+    const float mean = wave_sum(s) / (float)dim;
+    float q = 0.0f;
+    for (uint32_t i = lane; i < dim; i += kWave) {
+        const float d = Store<T>::load1(xin + i) - mean;
+        q = fmaf(d, d, q);
+    }
+    const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)dim + eps);
+    for (uint32_t i = lane; i < dim; i += kWave) {
+        const float t = (Store<T>::load1(xin + i) - mean) * rstd;
+        Store<T>::store1(yout + i, fmaf(t, gamma[i], beta[i]));
+    }
+}
+
+// ---- LayerNorm dispatch ----------------------------------------------------
+template <typename T, int NW, int VPL, int TL>
+void ln_launch(const T *x, T *y, const float *gamma, const float *beta, uint32_t rows, float eps,
+               float inv_dim, hipStream_t stream) {
+    constexpr uint32_t rows_per_block = (kWave / TL) * (kLnThreads / kWave);
+    const uint32_t blocks = (rows + rows_per_block - 1) / rows_per_block;
+    hipLaunchKernelGGL((ln_team_kernel<T, NW, VPL, TL>), dim3(blocks), dim3(kLnThreads), 0, stream, x,
+                       y, gamma, beta, rows, eps, inv_dim);
+}
+
+template <typename T, int NW, int TL>
+bool ln_launch_vpl(uint32_t vpl, const T *x, T *y, const float *gamma, const float *beta,
+                   uint32_t rows, float eps, float inv_dim, hipStream_t stream) {
+    switch (vpl) {
+        case 1: ln_launch<T, NW, 1, TL>(x, y, gamma, beta, rows, eps, inv_dim, stream); return true;
+        case 2: ln_launch<T, NW, 2, TL>(x, y, gamma, beta, rows, eps, inv_dim, stream); return true;
+        case 3: ln_launch<T, NW, 3, TL>(x, y, gamma, beta, rows, eps, inv_dim, stream); return true;
+        case 4: ln_launch<T, NW, 4, TL>(x, y, gamma, beta, rows, eps, inv_dim, stream); return true;
+        case 5: ln_launch<T, NW, 5, TL>(x, y, gamma, beta, rows, eps, inv_dim, stream); return true;
+        case 6: ln_launch<T, NW, 6, TL>(x, y, gamma, beta, rows, eps, inv_dim, stream); return true;
+        case 7: ln_launch<T, NW, 7, TL>(x, y, gamma, beta, rows, eps, inv_dim, stream); return true;
+        case 8: ln_launch<T, NW, 8, TL>(x, y, gamma, beta, rows, eps, inv_dim, stream); return true;
+        default: return false;
+    }
+}
+
+// Tries the team kernel with NW-dword chunks; false when the row does not decompose.
+template <typename T, int NW>
+bool ln_try(const T *x, T *y, const float *gamma, const float *beta, uint32_t rows, uint32_t dim,
+            float eps, float inv_dim, hipStream_t stream) {
+    constexpr uint32_t N = NW * 4 / sizeof(T);
+    if (dim % N != 0) return false;
+    const uint32_t chunks = dim / N;
+    uint32_t tl = kWave;
+    while (chunks % tl != 0) tl /= 2;
+    const uint32_t vpl = chunks / tl;
+    switch (tl) {
+        case 64: return ln_launch_vpl<T, NW, 64>(vpl, x, y, gamma, beta, rows, eps, inv_dim, stream);
+        case 32: return ln_launch_vpl<T, NW, 32>(vpl, x, y, gamma, beta, rows, eps, inv_dim, stream);
+        case 16: return ln_launch_vpl<T, NW, 16>(vpl, x, y, gamma, beta, rows, eps, inv_dim, stream);
+        case 8: return ln_launch_vpl<T, NW, 8>(vpl, x, y, gamma, beta, rows, eps, inv_dim, stream);
+        case 4: return ln_launch_vpl<T, NW, 4>(vpl, x, y, gamma, beta, rows, eps, inv_dim, stream);
+        default: return false;
+    }
+}
+
+}  // namespace
+
+int g_ln_chunk_override = 0;  // 0 = automatic, 8 or 16 = forced chunk bytes (tuning)
+
+template <typename T>
+int ln_dispatch(const void *xv, void *yv, const float *gamma, const float *beta, size_t rows,
+                size_t dim, float eps, hipStream_t stream) {
+    const T *x = static_cast<const T *>(xv);
+    T *y = static_cast<T *>(yv);
+    if (rows == 0 || dim == 0) return MSD_OK;
+    if (rows > 0x7FFFFFFFull || dim > 0x7FFFFFFFull) return MSD_ERR_INVALID_VALUE;
+    const float inv_dim = 1.0f / (float)dim;
+    const uint32_t r = (uint32_t)rows, d = (uint32_t)dim;
+    bool done = false;
+    if (aligned16(x) && aligned16(y) && aligned16(gamma) && aligned16(beta)) {
+        // A lane's dependent chain (convert, two reductions, affine) is on the critical path
+        // of a launch this short, so half-precision rows are spread over more lanes with
+        // 8-byte chunks when 16-byte ones would leave a team of fewer than 64 lanes with more
+        // than 16 elements per lane (measured 10-20 % faster at dim 320 / 640 / 1280); float
+        // rows keep 16-byte chunks (8-byte ones only add load instructions).
+        const uint32_t n16 = 16 / sizeof(T);
+        bool prefer8 = false;
+        if (sizeof(T) == 2 && d % n16 == 0) {
+            uint32_t tl = kWave;
+            while ((d / n16) % tl != 0) tl /= 2;
+            prefer8 = tl < kWave && (d / tl) > 16;
+        }
+        if (g_ln_chunk_override == 8) prefer8 = true;
+        if (g_ln_chunk_override == 16) prefer8 = false;
+        if (prefer8) done = ln_try<T, 2>(x, y, gamma, beta, r, d, eps, inv_dim, stream);
+        if (!done) done = ln_try<T, 4>(x, y, gamma, beta, r, d, eps, inv_dim, stream);
+        if (!done && !prefer8) done = ln_try<T, 2>(x, y, gamma, beta, r, d, eps, inv_dim, stream);
+    }
+    if (!done) {
+        const uint32_t rows_per_block = kLnThreads / kWave;
+        hipLaunchKernelGGL((ln_generic_kernel<T>),
+                           dim3((uint32_t)((rows + rows_per_block - 1) / rows_per_block)),
+                           dim3(kLnThreads), 0, stream, x, y, gamma, beta, (uint32_t)rows,
+                           (uint32_t)dim, eps);
+    }
+    return launch_status();
+}
+
+template int ln_dispatch<float>(const void *, void *, const float *, const float *, size_t, size_t,
+                                float, hipStream_t);
+template int ln_dispatch<__half>(const void *, void *, const float *, const float *, size_t, size_t,
+                                 float, hipStream_t);
+
+}  // namespace msd

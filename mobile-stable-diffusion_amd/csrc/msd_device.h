@@ -71,6 +71,15 @@ __device__ __forceinline__ void store_stream(u32x4 *p, const u32x4 &v) {
     __builtin_nontemporal_store(v, p);
 }
 
+// Makes the compiler forget what it knows about a packed vector held in registers, so
+// that conversions of it are redone where they are used instead of being kept live
+// (unpacked copies of a register-resident slice would not fit the register file).
+__device__ __forceinline__ void forget(u32x4 &v) {
+    uint32_t a = v[0], b = v[1], c = v[2], d = v[3];
+    asm volatile("" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+    v = u32x4{a, b, c, d};
+}
+
 // ---------------------------------------------------------------------------
 // Division by a launch-time constant d (n < 2^31): q = umulhi(n, mul) >> shift.
 // mul = ceil(2^(31+L) / d), shift = L-1 with L = ceil(log2 d), d >= 2; d == 1 is

@@ -1,0 +1,56 @@
+// Host-side declarations shared by the translation units of libmsd_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/msd_hip.h"
+
+namespace msd {
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline int launch_status() { return (int)hipGetLastError(); }
+
+// ---- GroupNorm scratch: what workgroups sharing one (sample, group) exchange ----
+constexpr uint32_t kGnMaxSplit = 64;    // workgroups per unit (one wavefront reads all slots)
+constexpr uint32_t kGnMaxUnits = 8192;  // units that own scratch slots; larger launches never split
+
+struct GnScratch {
+    unsigned long long *slot_mean;  // [kGnMaxUnits][kGnMaxSplit]  (tag << 32) | float bits
+    unsigned long long *slot_m2;    // [kGnMaxUnits][kGnMaxSplit]
+    uint32_t *epoch;                // [kGnMaxUnits] launches completed on this unit
+    uint32_t *done;                 // [kGnMaxUnits] slices finished in the running launch
+    uint32_t *status;               // [1] sticky: bit 0 = a wait ran out of polls
+};
+
+// Per-(device, stream) scratch, created on first use (hipMalloc + hipMemset).
+hipError_t get_scratch(hipStream_t stream, GnScratch *out);
+
+// Forced launch plan for msd_groupnorm (0 = choose automatically).
+struct GnPlanOverride {
+    int split;
+    int threads;
+};
+extern GnPlanOverride g_gn_plan_override;
+extern int g_ln_chunk_override;  // 0 = automatic, 8 / 16 = forced LayerNorm chunk bytes
+
+// ---- per-dtype dispatchers (T = float or __half), defined in the kernel files ----
+template <typename T>
+int gn_dispatch(const void *x, void *y, const float *gamma, const float *beta, size_t batch,
+                size_t channels, size_t hw, size_t groups, float eps, bool silu,
+                hipStream_t stream);
+template <typename T>
+int ln_dispatch(const void *x, void *y, const float *gamma, const float *beta, size_t rows,
+                size_t dim, float eps, hipStream_t stream);
+template <typename T>
+int geglu_dispatch(const void *proj, void *out, size_t rows, size_t inner, hipStream_t stream);
+
+enum class Act { Silu, Gelu, QuickGelu };
+template <typename T>
+int act_dispatch(Act op, const void *x, void *y, size_t n, hipStream_t stream);
+template <typename T>
+int temb_dispatch(const int64_t *timesteps, void *out, size_t batch, size_t dim, float max_period,
+                  hipStream_t stream);
+
+}  // namespace msd

@@ -1,0 +1,228 @@
+// Streaming kernels for gfx950: the GEGLU epilogue, elementwise SiLU / GELU /
+// quick_GELU and the sinusoidal timestep embedding.  Flat 16-byte accesses, U
+// vectors per lane with every load issued before the first use; all workgroups
+// but a ragged last one run branch-free.
+#include "msd_device.h"
+#include "msd_internal.h"
+
+#include <cmath>
+
+namespace msd {
+namespace {
+
+FastDiv make_fast_div(uint32_t d) {
+    FastDiv fd{0u, 0u, d};
+    if (d <= 1) return fd;
+    uint32_t L = 0;
+    while ((1ull << L) < d) L++;
+    fd.mul = (uint32_t)(((1ull << (31 + L)) + d - 1) / d);
+    fd.shift = L - 1;
+    return fd;
+}
+
+constexpr int kStreamThreads = 256;
+constexpr int kStreamUnroll = 4;
+
+// out[r, c] = proj[r, c] * gelu(proj[r, inner + c]); vectors never straddle a row.
+// Every workgroup but the last takes the branch-free path: 2*U loads in flight
+// per lane before the first use.
+template <typename T>
+__global__ __launch_bounds__(kStreamThreads) void geglu_kernel(const T *__restrict__ proj,
+                                                               T *__restrict__ out,
+                                                               uint32_t out_vecs,
+                                                               FastDiv vec_per_row) {
+    constexpr int EPV = Store<T>::EPV;
+    constexpr int U = kStreamUnroll;
+    const u32x4 *in = reinterpret_cast<const u32x4 *>(proj);
+    u32x4 *o = reinterpret_cast<u32x4 *>(out);
+    const uint32_t block_base = blockIdx.x * (kStreamThreads * U);
+    const uint32_t base = block_base + threadIdx.x;
+    const bool full = block_base + kStreamThreads * U <= out_vecs;  // uniform
+    u32x4 va[U], vb[U];
+    uint32_t ovs[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const uint32_t ov = base + u * kStreamThreads;
+        ovs[u] = full ? ov : min(ov, out_vecs - 1);  // ragged last block re-reads the last vector
+        const uint32_t r = fast_div(ovs[u], vec_per_row);
+        const size_t iv = (size_t)ovs[u] + (size_t)r * vec_per_row.d;  // r*2*vpr + (ov - r*vpr)
+        va[u] = load_stream(in + iv);
+        vb[u] = load_stream(in + iv + vec_per_row.d);
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        float a[EPV], b[EPV], r[EPV];
+        Store<T>::unpack(va[u], a);
+        Store<T>::unpack(vb[u], b);
+#pragma unroll
+        for (int e = 0; e < EPV; e++) r[e] = a[e] * gelu_erf_f(b[e]);
+        const u32x4 packed = Store<T>::pack(r);
+        if (full || base + u * kStreamThreads < out_vecs) store_stream(o + ovs[u], packed);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kStreamThreads) void geglu_generic_kernel(
+    const T *__restrict__ proj, T *__restrict__ out, size_t rows, size_t inner) {
+    const size_t n = rows * inner;
+    for (size_t i = (size_t)blockIdx.x * kStreamThreads + threadIdx.x; i < n;
+         i += (size_t)gridDim.x * kStreamThreads) {
+        const size_t r = i / inner, c = i - r * inner;
+        const float a = Store<T>::load1(proj + r * 2 * inner + c);
+        const float b = Store<T>::load1(proj + r * 2 * inner + inner + c);
+        Store<T>::store1(out + i, a * gelu_erf_f(b));
+    }
+}
+
+// y[i] = OP(x[i]); y may alias x: a lane reads its vectors before it writes them,
+// and in the ragged last block the duplicated reads are never written back.
+template <typename T, typename OP>
+__global__ __launch_bounds__(kStreamThreads) void act_kernel(const T *x, T *y, uint32_t vecs,
+                                                             size_t n) {
+    constexpr int EPV = Store<T>::EPV;
+    constexpr int U = kStreamUnroll;
+    const u32x4 *in = reinterpret_cast<const u32x4 *>(x);
+    u32x4 *o = reinterpret_cast<u32x4 *>(y);
+    const uint32_t block_base = blockIdx.x * (kStreamThreads * U);
+    const uint32_t base = block_base + threadIdx.x;
+    const bool full = block_base + kStreamThreads * U <= vecs;  // uniform
+    if (vecs != 0) {
+        u32x4 raw[U];
+        uint32_t vs[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint32_t v = base + u * kStreamThreads;
+            vs[u] = full ? v : min(v, vecs - 1);
+            raw[u] = load_stream(in + vs[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            float f[EPV];
+            Store<T>::unpack(raw[u], f);
+#pragma unroll
+            for (int e = 0; e < EPV; e++) f[e] = OP::apply(f[e]);
+            const u32x4 packed = Store<T>::pack(f);
+            if (full || base + u * kStreamThreads < vecs) store_stream(o + vs[u], packed);
+        }
+    }
+    // ragged tail (n % EPV elements) by the first lanes of block 0
+    const size_t tail = (size_t)vecs * EPV;
+    if (blockIdx.x == 0 && tail + threadIdx.x < n)
+        Store<T>::store1(y + tail + threadIdx.x,
+                         OP::apply(Store<T>::load1(x + tail + threadIdx.x)));
+}
+
+template <typename T, typename OP>
+__global__ __launch_bounds__(kStreamThreads) void act_generic_kernel(const T *x, T *y, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * kStreamThreads + threadIdx.x; i < n;
+         i += (size_t)gridDim.x * kStreamThreads)
+        Store<T>::store1(y + i, OP::apply(Store<T>::load1(x + i)));
+}
+
+// ---------------------------------------------------------------------------
+// Timestep embedding
+// ---------------------------------------------------------------------------
+// freq_i is the float32 expression exp(neg_log_period * float(i) / float(half))
+// with one rounding per operation; exp is evaluated in double and rounded once,
+// which reproduces a correctly rounded float exp.  The angle float(t)*freq is a
+// single float32 product; cos / sin are evaluated in double and rounded once.
+template <typename T>
+__global__ __launch_bounds__(256) void timestep_embedding_kernel(
+    const int64_t *__restrict__ timesteps, T *__restrict__ out, uint32_t batch, uint32_t half,
+    float neg_log_period) {
+    const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= batch * half) return;
+    const uint32_t b = idx / half, i = idx - b * half;
+    const float z = __fdiv_rn(__fmul_rn(neg_log_period, (float)i), (float)half);
+    const float freq = (float)exp((double)z);
+    const float arg = __fmul_rn((float)timesteps[b], freq);
+    double sn, cs;
+    sincos((double)arg, &sn, &cs);
+    T *row = out + (size_t)b * (2 * half);
+    Store<T>::store1(row + i, (float)cs);
+    Store<T>::store1(row + half + i, (float)sn);
+}
+
+// ---- streaming dispatch ----------------------------------------------------
+inline uint32_t stream_blocks(size_t vecs) {
+    const size_t per_block = (size_t)kStreamThreads * kStreamUnroll;
+    return (uint32_t)((vecs + per_block - 1) / per_block);
+}
+
+}  // namespace
+
+template <typename T>
+int geglu_dispatch(const void *pv, void *ov, size_t rows, size_t inner, hipStream_t stream) {
+    constexpr int EPV = Store<T>::EPV;
+    const T *proj = static_cast<const T *>(pv);
+    T *out = static_cast<T *>(ov);
+    if (rows == 0 || inner == 0) return MSD_OK;
+    const size_t out_vecs = rows * (inner / EPV);
+    if (aligned16(proj) && aligned16(out) && inner % EPV == 0 && out_vecs < 0x7FFFFFFFull &&
+        rows < 0x7FFFFFFFull) {
+        hipLaunchKernelGGL((geglu_kernel<T>), dim3(stream_blocks(out_vecs)), dim3(kStreamThreads),
+                           0, stream, proj, out, (uint32_t)out_vecs,
+                           make_fast_div((uint32_t)(inner / EPV)));
+    } else {
+        const size_t n = rows * inner;
+        const size_t want = (n + kStreamThreads - 1) / kStreamThreads;
+        hipLaunchKernelGGL((geglu_generic_kernel<T>), dim3((uint32_t)(want < 65536 ? want : 65536)),
+                           dim3(kStreamThreads), 0, stream, proj, out, rows, inner);
+    }
+    return launch_status();
+}
+
+namespace {
+
+template <typename T, typename OP>
+int act_launch(const void *xv, void *yv, size_t n, hipStream_t stream) {
+    constexpr int EPV = Store<T>::EPV;
+    const T *x = static_cast<const T *>(xv);
+    T *y = static_cast<T *>(yv);
+    if (n == 0) return MSD_OK;
+    const size_t vecs = n / EPV;
+    if (aligned16(x) && aligned16(y) && vecs < 0x7FFFFFFFull) {
+        const uint32_t blocks = vecs ? stream_blocks(vecs) : 1u;
+        hipLaunchKernelGGL((act_kernel<T, OP>), dim3(blocks), dim3(kStreamThreads), 0, stream, x, y,
+                           (uint32_t)vecs, n);
+    } else {
+        const size_t want = (n + kStreamThreads - 1) / kStreamThreads;
+        hipLaunchKernelGGL((act_generic_kernel<T, OP>),
+                           dim3((uint32_t)(want < 65536 ? want : 65536)), dim3(kStreamThreads), 0,
+                           stream, x, y, n);
+    }
+    return launch_status();
+}
+
+
+}  // namespace
+
+template <typename T>
+int act_dispatch(Act op, const void *x, void *y, size_t n, hipStream_t stream) {
+    switch (op) {
+        case Act::Silu: return act_launch<T, OpSilu>(x, y, n, stream);
+        case Act::Gelu: return act_launch<T, OpGelu>(x, y, n, stream);
+        case Act::QuickGelu: return act_launch<T, OpQuickGelu>(x, y, n, stream);
+    }
+    return MSD_ERR_INVALID_VALUE;
+}
+
+template <typename T>
+int temb_dispatch(const int64_t *timesteps, void *out, size_t batch, size_t dim, float max_period,
+                  hipStream_t stream) {
+    const uint32_t half = (uint32_t)(dim / 2);
+    const uint32_t blocks = (uint32_t)((batch * half + 255) / 256);
+    const float neg_log_period = -logf(max_period);  // host float log, as in the replaced host loop
+    hipLaunchKernelGGL((timestep_embedding_kernel<T>), dim3(blocks), dim3(256), 0, stream, timesteps,
+                       static_cast<T *>(out), (uint32_t)batch, half, neg_log_period);
+    return launch_status();
+}
+
+template int geglu_dispatch<float>(const void *, void *, size_t, size_t, hipStream_t);
+template int geglu_dispatch<__half>(const void *, void *, size_t, size_t, hipStream_t);
+template int act_dispatch<float>(Act, const void *, void *, size_t, hipStream_t);
+template int act_dispatch<__half>(Act, const void *, void *, size_t, hipStream_t);
+template int temb_dispatch<float>(const int64_t *, void *, size_t, size_t, float, hipStream_t);
+template int temb_dispatch<__half>(const int64_t *, void *, size_t, size_t, float, hipStream_t);
+
+}  // namespace msd

@@ -69,7 +69,9 @@ def test_argument_validation_needs_no_gpu(msd):
     assert lib.msd_geglu(None, None, 4, 64, 0, None) == 1
     assert lib.msd_silu(None, None, 4, 0, None) == 1
     assert lib.msd_timestep_embedding(None, None, 2, 321, 10000.0, 0, None) == 1
-    assert lib.msd_set_groupnorm_target_blocks(0) == 1
+    assert lib.msd_set_groupnorm_plan(3, 0) == 1
+    assert lib.msd_set_groupnorm_plan(0, 100) == 1
+    assert lib.msd_set_groupnorm_plan(0, 0) == 0
 
 
 def test_missing_library_fails_loudly(msd):

@@ -89,29 +89,36 @@ def test_groupnorm_in_place_and_no_silu(msd, orc, cuda, half):
     _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-6, False, half)
 
 
-@pytest.mark.parametrize("target_blocks", [1, 64, 2048, 8192])
-def test_groupnorm_every_split_factor(msd, orc, cuda, target_blocks):
+@pytest.mark.parametrize("split,threads", [(1, 0), (2, 0), (4, 0), (8, 256), (16, 0), (64, 64), (2, 1024),
+                                           (4, 320), (1, 640)])
+def test_groupnorm_every_split_factor(msd, orc, cuda, split, threads):
     # the same tensor through 1 .. 64 workgroups per group must agree with the oracle
     lib = msd.load_library()
     x = orc.normal((2, 320, 64, 64), seed=88, sigma=2.0, mean=1.0)
     g, b = _affine(orc, 320, 88)
     try:
-        assert lib.msd_set_groupnorm_target_blocks(target_blocks) == 0
+        assert lib.msd_set_groupnorm_plan(split, threads) == 0
         for half in (False, True):
             _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half)
+            _run_groupnorm(msd, orc, cuda, x[:1, :96, :24, :24].copy(), g[:96], b[:96], 32, 1e-5, True, half)
     finally:
-        lib.msd_set_groupnorm_target_blocks(512)
+        lib.msd_set_groupnorm_plan(0, 0)
     assert msd.status() == 0
 
 
 def test_groupnorm_repeated_launches_reuse_scratch(msd, orc, cuda):
     # the arrival counters are never reset: many launches with changing split factors
+    lib = msd.load_library()
     shapes = [(2, 320, 4096), (2, 1280, 64), (1, 640, 1024), (2, 1920, 256), (2, 320, 4096)]
-    for rep in range(3):
-        for i, shp in enumerate(shapes):
-            x = orc.normal(shp, seed=900 + i + 10 * rep, sigma=2.0)
-            g, b = _affine(orc, shp[1], 900 + i)
-            _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half=True)
+    try:
+        for rep in range(3):
+            for i, shp in enumerate(shapes):
+                lib.msd_set_groupnorm_plan([4, 2, 8, 1][(rep + i) % 4], 0)
+                x = orc.normal(shp, seed=900 + i + 10 * rep, sigma=2.0)
+                g, b = _affine(orc, shp[1], 900 + i)
+                _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half=True)
+    finally:
+        lib.msd_set_groupnorm_plan(0, 0)
     assert msd.status() == 0
 
 
@@ -216,6 +223,26 @@ def test_layernorm_dims_and_ragged_rows(msd, orc, cuda, rows, dim, half):
         assert_close_f16(got, orc.round_to_half(ref.astype(np.float32)), "ln dims f16")
     else:
         assert_close_f32(got, ref, what="ln dims f32")
+
+
+@pytest.mark.parametrize("chunk", [8, 16])
+def test_layernorm_forced_chunk_width(msd, orc, cuda, chunk):
+    lib = msd.load_library()
+    try:
+        assert lib.msd_set_layernorm_chunk(chunk) == 0
+        for rows, dim, half in [(8192, 320, True), (300, 640, True), (77, 768, False), (33, 1280, False),
+                                (5, 64, True), (5, 64, False), (9, 2048, True)]:
+            x = orc.normal((rows, dim), seed=rows + dim + chunk, sigma=1.5, mean=-1.0)
+            xin = orc.round_to_half(x) if half else x
+            g, b = _affine(orc, dim, dim + 1)
+            ref = orc.layernorm(xin, g, b, 1e-5)
+            got = msd.layernorm(_to_dev(xin, cuda, half), _to_dev(g, cuda), _to_dev(b, cuda)).float().cpu().numpy()
+            if half:
+                assert_close_f16(got, orc.round_to_half(ref), "ln chunk f16")
+            else:
+                assert_close_f32(got, ref, what="ln chunk f32")
+    finally:
+        lib.msd_set_layernorm_chunk(0)
 
 
 def test_layernorm_in_place_fixtures_and_empty(msd, orc, golden, cuda):
