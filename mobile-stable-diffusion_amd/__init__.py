@@ -170,3 +170,65 @@ def ddim_timesteps(steps):
     buf = (ctypes.c_int * n)()
     lib.msd_ddim_timesteps(steps, buf, n)
     return list(buf)
+
+
+# ---------------------------------------------------------------------------------------
+# C++ layer objects (libmsd_nn.so) through their plain-C handles
+# ---------------------------------------------------------------------------------------
+_nn = None
+
+
+def load_nn_library(path=None):
+    """Loads libmsd_nn.so (GroupNorm / LayerNorm / GEGLU objects, NPY loader, step runner)."""
+    global _nn
+    if _nn is not None and path is None:
+        return _nn
+    load_library()
+    path = path or LIB_NN_PATH
+    if not os.path.exists(path):
+        raise MsdError("native library %s is missing: run __graft_entry__.build()" % path)
+    nn = ctypes.CDLL(path)
+    vp, sz, fl, it, cp = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float, ctypes.c_int, ctypes.c_char_p
+    szp = ctypes.POINTER(ctypes.c_size_t)
+    flp = ctypes.POINTER(ctypes.c_float)
+    lgp = ctypes.POINTER(ctypes.c_long)
+    sig = {
+        "msdnn_last_error": (cp, []),
+        "msdnn_set_media_path": (None, [cp]),
+        "msdnn_npy_load": (it, [cp, flp, sz, szp, szp]),
+        "msdnn_npy_save": (it, [cp, flp, sz]),
+        "msdnn_groupnorm_create": (vp, [vp, sz, sz, fl, cp, cp, sz, it]),
+        "msdnn_groupnorm_init": (it, [vp]),
+        "msdnn_groupnorm_check": (it, [vp, sz, it]),
+        "msdnn_groupnorm_forward": (it, [vp, vp, vp, sz, it]),
+        "msdnn_groupnorm_destroy": (None, [vp]),
+        "msdnn_layernorm_create": (vp, [vp, sz, cp, cp, fl]),
+        "msdnn_layernorm_init": (it, [vp]),
+        "msdnn_layernorm_check": (it, [vp, sz, it]),
+        "msdnn_layernorm_forward": (it, [vp, vp, vp, sz, it]),
+        "msdnn_layernorm_destroy": (None, [vp]),
+        "msdnn_geglu_create": (vp, [vp, sz, sz]),
+        "msdnn_geglu_weight_shape": (it, [vp, szp, szp]),
+        "msdnn_geglu_check": (it, [vp, sz, sz, it]),
+        "msdnn_geglu_forward": (it, [vp, vp, sz, vp, sz, it]),
+        "msdnn_geglu_destroy": (None, [vp]),
+        "msdnn_activation": (it, [vp, it, vp, vp, sz, it]),
+        "msdnn_timestep_embedding": (it, [vp, lgp, sz, flp]),
+        "msdnn_ddim_timesteps": (it, [it, ctypes.POINTER(ctypes.c_int), it]),
+        "msdnn_test_buffer": (it, [vp, vp, sz, it, cp, flp, szp]),
+        "msdnn_step_create": (vp, [vp, sz, it]),
+        "msdnn_step_bytes": (sz, [vp]),
+        "msdnn_step_launches": (sz, [vp]),
+        "msdnn_step_run": (it, [vp, it, it, lgp, sz]),
+        "msdnn_step_destroy": (None, [vp]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(nn, name)
+        fn.restype = res
+        fn.argtypes = args
+    _nn = nn
+    return nn
+
+
+def nn_last_error():
+    return load_nn_library().msdnn_last_error().decode()

@@ -60,12 +60,12 @@ def build_nn():
     srcs = sorted(os.path.join(nn_dir, f) for f in os.listdir(nn_dir) if f.endswith(".cpp"))
     if not srcs:
         return None
-    # host-only C++; hipcc is used for the HIP runtime include / link paths
-    cmd = [HIPCC, "-O2", "-std=c++17", "-fPIC", "-shared", "-x", "c++",
-           "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(REPO, "include"), "-I", nn_dir,
-           "-Wall", "-Wno-unused-command-line-argument"] + srcs + [
-           "-o", LIB_NN, "-L", CSRC, "-lmsd_hip", "-Wl,-rpath,$ORIGIN", "-lamdhip64",
-           "-L/opt/rocm/lib"]
+    # host-only C++ against the HIP runtime API: the system compiler, no device code
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared",
+           "-D__HIP_PLATFORM_AMD__", "-I", "/opt/rocm/include", "-I", os.path.join(REPO, "include"),
+           "-I", nn_dir, "-Wall", "-Wno-deprecated-declarations"] + srcs + [
+           "-o", LIB_NN, "-L", CSRC, "-lmsd_hip", "-L/opt/rocm/lib", "-lamdhip64",
+           "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"]
     _run(cmd)
     return LIB_NN
 

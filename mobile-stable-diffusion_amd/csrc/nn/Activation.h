@@ -1,0 +1,19 @@
+// Elementwise activations.  In the reference these are not objects: a caller sets the two
+// arguments of utilKernel->silu / utilKernel->gelu and enqueues it over the element count
+// (M/nn/ResBlock.cpp:136-142, M/nn/ResidualAttentionBlock.cpp:146-153).  The equivalents
+// take source and destination buffers (the same buffer for the in-place call sites).
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+
+#include "DeviceBuffer.h"
+
+namespace msd {
+
+// Each returns 0 or a hipError_t value and throws std::runtime_error when dst and src differ
+// in size or storage type.
+int silu(hipStream_t stream, const DeviceBuffer &src, DeviceBuffer &dst);        // K/util.cl:124-134
+int gelu(hipStream_t stream, const DeviceBuffer &src, DeviceBuffer &dst);        // K/util.cl:104-122
+int quick_gelu(hipStream_t stream, const DeviceBuffer &src, DeviceBuffer &dst);  // x*sigmoid(1.702x)
+
+}  // namespace msd

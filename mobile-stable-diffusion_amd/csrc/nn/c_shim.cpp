@@ -1,0 +1,216 @@
+// Plain-C handles over the C++ layer objects, for callers that cannot bind C++ (the tests
+// drive the objects through these with ctypes; a JNI or cgo stub would bind the same
+// functions).  Every function returns 0 on success; a negative value means a C++ exception
+// was caught and msdnn_last_error() holds its text (the layer objects throw
+// std::runtime_error where the reference does); a positive value is a hipError_t.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+#include <exception>
+#include <string>
+
+#include "Activation.h"
+#include "GEGLU.h"
+#include "GroupNorm.h"
+#include "LayerNorm.h"
+#include "TimestepEmbedding.h"
+#include "UNetNormActStep.h"
+#include "util.h"
+
+using namespace msd;
+
+namespace {
+thread_local std::string g_last_error;
+
+template <typename F>
+int guarded(F f) {
+    try {
+        return f();
+    } catch (const std::exception &e) {
+        g_last_error = e.what();
+        return -1;
+    } catch (...) {
+        g_last_error = "unknown exception";
+        return -1;
+    }
+}
+
+DeviceBuffer wrap(void *p, size_t bytes, int dtype) {
+    return DeviceBuffer(p, bytes, dtype == MSD_DTYPE_F16 ? DType::F16 : DType::F32);
+}
+}  // namespace
+
+extern "C" {
+
+const char *msdnn_last_error(void) { return g_last_error.c_str(); }
+
+void msdnn_set_media_path(const char *dir) { util::setMediaPath(dir ? dir : ""); }
+
+// ---- npy (host only)
+int msdnn_npy_load(const char *name, float *out, size_t cap, size_t *num_vals, size_t *ndim) {
+    return guarded([&] {
+        const npy::Array a = util::load_npy_file(name);
+        if (num_vals) *num_vals = a.num_vals();
+        if (ndim) *ndim = a.shape.size();
+        if (out) memcpy(out, a.data.data(), sizeof(float) * (a.num_vals() < cap ? a.num_vals() : cap));
+        return 0;
+    });
+}
+int msdnn_npy_save(const char *path, const float *data, size_t n) {
+    return guarded([&] {
+        npy::save(path, {n}, data);
+        return 0;
+    });
+}
+
+// ---- GroupNorm
+void *msdnn_groupnorm_create(void *stream, size_t num_groups, size_t num_channels, float eps,
+                             const char *weight_name, const char *bias_name, size_t batch, int fuse_silu) {
+    GroupNorm *g = nullptr;
+    guarded([&] {
+        g = new GroupNorm(static_cast<hipStream_t>(stream), num_groups, num_channels, eps, weight_name,
+                          bias_name, batch, fuse_silu != 0);
+        return 0;
+    });
+    return g;
+}
+int msdnn_groupnorm_init(void *h) {
+    return guarded([&] {
+        static_cast<GroupNorm *>(h)->init();
+        return 0;
+    });
+}
+int msdnn_groupnorm_check(void *h, size_t input_bytes, int dtype) {
+    return guarded([&] {
+        static_cast<GroupNorm *>(h)->checkInput(input_bytes, dtype == MSD_DTYPE_F16 ? DType::F16 : DType::F32);
+        return 0;
+    });
+}
+int msdnn_groupnorm_forward(void *h, void *in, void *out, size_t bytes, int dtype) {
+    return guarded([&] {
+        DeviceBuffer i = wrap(in, bytes, dtype), o = wrap(out, bytes, dtype);
+        return static_cast<GroupNorm *>(h)->forward(i, o);
+    });
+}
+void msdnn_groupnorm_destroy(void *h) { delete static_cast<GroupNorm *>(h); }
+
+// ---- LayerNorm
+void *msdnn_layernorm_create(void *stream, size_t dim, const char *weight_name, const char *bias_name,
+                             float eps) {
+    LayerNorm *l = nullptr;
+    guarded([&] {
+        l = new LayerNorm(static_cast<hipStream_t>(stream), dim, weight_name, bias_name, eps);
+        return 0;
+    });
+    return l;
+}
+int msdnn_layernorm_init(void *h) {
+    return guarded([&] {
+        static_cast<LayerNorm *>(h)->init();
+        return 0;
+    });
+}
+int msdnn_layernorm_check(void *h, size_t input_bytes, int dtype) {
+    return guarded([&] {
+        static_cast<LayerNorm *>(h)->checkInput(input_bytes, dtype == MSD_DTYPE_F16 ? DType::F16 : DType::F32);
+        return 0;
+    });
+}
+int msdnn_layernorm_forward(void *h, void *in, void *out, size_t bytes, int dtype) {
+    return guarded([&] {
+        DeviceBuffer i = wrap(in, bytes, dtype), o = wrap(out, bytes, dtype);
+        return static_cast<LayerNorm *>(h)->forward(i, o);
+    });
+}
+void msdnn_layernorm_destroy(void *h) { delete static_cast<LayerNorm *>(h); }
+
+// ---- GEGLU
+void *msdnn_geglu_create(void *stream, size_t in_features, size_t out_features) {
+    return new GEGLU(static_cast<hipStream_t>(stream), in_features, out_features);
+}
+int msdnn_geglu_weight_shape(void *h, size_t *rows, size_t *cols) {
+    *rows = static_cast<GEGLU *>(h)->weightShape[0];
+    *cols = static_cast<GEGLU *>(h)->weightShape[1];
+    return 0;
+}
+int msdnn_geglu_check(void *h, size_t in_bytes, size_t out_bytes, int dtype) {
+    return guarded([&] {
+        static_cast<GEGLU *>(h)->checkInput(in_bytes, out_bytes, dtype == MSD_DTYPE_F16 ? DType::F16 : DType::F32);
+        return 0;
+    });
+}
+int msdnn_geglu_forward(void *h, void *in, size_t in_bytes, void *out, size_t out_bytes, int dtype) {
+    return guarded([&] {
+        DeviceBuffer i = wrap(in, in_bytes, dtype), o = wrap(out, out_bytes, dtype);
+        return static_cast<GEGLU *>(h)->forward(i, o);
+    });
+}
+void msdnn_geglu_destroy(void *h) { delete static_cast<GEGLU *>(h); }
+
+// ---- activations: op 0 silu, 1 gelu, 2 quick_gelu
+int msdnn_activation(void *stream, int op, void *src, void *dst, size_t bytes, int dtype) {
+    return guarded([&] {
+        DeviceBuffer s = wrap(src, bytes, dtype), d = wrap(dst, bytes, dtype);
+        hipStream_t st = static_cast<hipStream_t>(stream);
+        return op == 0 ? silu(st, s, d) : op == 1 ? gelu(st, s, d) : quick_gelu(st, s, d);
+    });
+}
+
+// ---- timestep embedding: writes batch*dim floats to host memory `out`
+int msdnn_timestep_embedding(void *stream, const long *timesteps, size_t batch, float *out) {
+    return guarded([&] {
+        hipStream_t st = static_cast<hipStream_t>(stream);
+        DeviceBuffer e = createTimestepEmbedding(st, std::vector<long>(timesteps, timesteps + batch));
+        const std::vector<float> host = util::download(e, st);
+        memcpy(out, host.data(), host.size() * sizeof(float));
+        return 0;
+    });
+}
+int msdnn_ddim_timesteps(int steps, int *out, int cap) {
+    int n = 0;
+    const int rc = guarded([&] {
+        const std::vector<int> t = ddimTimesteps(steps);
+        n = (int)t.size();
+        for (int i = 0; i < n && i < cap; i++) out[i] = t[(size_t)i];
+        return 0;
+    });
+    return rc < 0 ? rc : n;
+}
+
+// ---- golden-file comparison (util::testBuffer)
+int msdnn_test_buffer(void *stream, void *ptr, size_t bytes, int dtype, const char *golden, float *max_diff,
+                      size_t *num_wrong) {
+    return guarded([&] {
+        const util::TestResult r =
+            util::testBuffer(static_cast<hipStream_t>(stream), wrap(ptr, bytes, dtype), golden);
+        if (max_diff) *max_diff = r.max_diff;
+        if (num_wrong) *num_wrong = r.num_wrong;
+        return r.size_matches ? 0 : -2;
+    });
+}
+
+// ---- one UNet step of the path
+void *msdnn_step_create(void *stream, size_t batch, int dtype) {
+    UNetNormActStep *s = nullptr;
+    guarded([&] {
+        s = new UNetNormActStep(static_cast<hipStream_t>(stream), batch,
+                                dtype == MSD_DTYPE_F16 ? DType::F16 : DType::F32);
+        return 0;
+    });
+    return s;
+}
+size_t msdnn_step_bytes(void *h) { return static_cast<UNetNormActStep *>(h)->bytesPerStep(); }
+size_t msdnn_step_launches(void *h) { return static_cast<UNetNormActStep *>(h)->launchesPerStep(); }
+// runs `steps` steps; graph != 0 replays one captured HIP graph per step
+int msdnn_step_run(void *h, int steps, int graph, const long *timesteps, size_t batch) {
+    return guarded([&] {
+        UNetNormActStep *s = static_cast<UNetNormActStep *>(h);
+        const std::vector<long> t(timesteps, timesteps + batch);
+        int rc = 0;
+        for (int i = 0; i < steps && rc == 0; i++) rc = graph ? s->forwardGraph() : s->forward(t);
+        return rc;
+    });
+}
+void msdnn_step_destroy(void *h) { delete static_cast<UNetNormActStep *>(h); }
+
+}  // extern "C"
