@@ -70,6 +70,12 @@ int msd_set_groupnorm_plan(int split, int threads);
 int msd_set_layernorm_chunk(int bytes);
 
 /*
+ * Tuning / test knob: 16-byte vectors each lane of msd_geglu produces (1, 2 or 4;
+ * 0 = automatic).  Process-wide.
+ */
+int msd_set_geglu_unroll(int vectors);
+
+/*
  * GroupNorm over NCHW, optionally followed by SiLU, in one launch.
  * Replaces the 3-kernel chain enqueued by GroupNorm::forward
  * (M/nn/GroupNorm.cpp:105-145; K/group_norm.cl:1-76) and, with fuse_silu != 0,

@@ -126,6 +126,12 @@ int msd_set_groupnorm_plan(int split, int threads) {
     return MSD_OK;
 }
 
+int msd_set_geglu_unroll(int vectors) {
+    if (vectors != 0 && vectors != 1 && vectors != 2 && vectors != 4) return MSD_ERR_INVALID_VALUE;
+    g_geglu_unroll_override = vectors;
+    return MSD_OK;
+}
+
 int msd_set_layernorm_chunk(int bytes) {
     if (bytes != 0 && bytes != 8 && bytes != 16) return MSD_ERR_INVALID_VALUE;
     g_ln_chunk_override = bytes;

@@ -33,6 +33,7 @@ struct GnPlanOverride {
     int threads;
 };
 extern GnPlanOverride g_gn_plan_override;
+extern int g_geglu_unroll_override;  // 0 = automatic, 1 / 2 / 4 = forced vectors per lane
 extern int g_ln_chunk_override;  // 0 = automatic, 8 / 16 = forced LayerNorm chunk bytes
 
 // ---- per-dtype dispatchers (T = float or __half), defined in the kernel files ----

@@ -280,6 +280,19 @@ def test_geglu_shapes_fp32_fp16(msd, orc, golden, cuda, rows, inner, half):
         assert_close_f32(msd.geglu(_to_dev(golden["geglu_proj"], cuda)).cpu().numpy(), golden["geglu_y"])
 
 
+@pytest.mark.parametrize("unroll", [1, 2, 4])
+def test_geglu_forced_vectors_per_lane(msd, orc, cuda, unroll):
+    lib = msd.load_library()
+    try:
+        assert lib.msd_set_geglu_unroll(unroll) == 0
+        for rows, inner in [(2048, 2560), (77, 1288), (3, 8), (1000, 24)]:
+            proj = orc.round_to_half(orc.normal((rows, 2 * inner), seed=rows + unroll, sigma=1.5))
+            got = msd.geglu(_to_dev(proj, cuda, True)).float().cpu().numpy()
+            assert_close_f16(got, orc.round_to_half(orc.geglu(proj)), "geglu unroll")
+    finally:
+        lib.msd_set_geglu_unroll(0)
+
+
 @pytest.mark.parametrize("name", ["silu", "gelu", "quick_gelu"])
 @pytest.mark.parametrize("half", [False, True], ids=["f32", "f16"])
 def test_activations(msd, orc, golden, cuda, name, half):
