@@ -298,19 +298,20 @@ def cpu_baseline(total_bytes, budget_s=12.0):
         return ()
 
     layers = step_layers()
-    # one untimed pass sizes the repetition count
-    t0 = time.perf_counter()
-    for kind, p in layers[:40]:
-        run(kind, p, make(kind, p))
-    est_step = (time.perf_counter() - t0) * len(layers) / 40.0
-    reps = max(1, min(50, int(budget_s / max(est_step, 1e-3))))
-    t_total = 0.0
-    for kind, p in layers:
-        data = make(kind, p)
-        t0 = time.perf_counter()
-        for _ in range(reps):
-            run(kind, p, data)
-        t_total += time.perf_counter() - t0
+
+    def timed_pass(reps):
+        total = 0.0
+        for kind, p in layers:
+            data = make(kind, p)
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                run(kind, p, data)
+            total += time.perf_counter() - t0
+        return total
+
+    probe = timed_pass(1)  # also warms the thread pool; sizes the timed pass
+    reps = max(2, min(400, int(budget_s / max(probe, 1e-3))))
+    t_total = timed_pass(reps)
     per_step = t_total / reps
     return {"value": round(total_bytes / per_step / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
             "ms_per_step": round(per_step * 1e3, 2), "seconds_timed": round(t_total, 2),

@@ -56,24 +56,16 @@ int msd_shutdown(void);
 int msd_status(void *stream);
 
 /*
- * Tuning / test knob: forces how msd_groupnorm cuts each (sample, group) into
- * workgroups.  split = workgroups per group (power of two <= 64, 0 = automatic;
- * a value below what fits in registers is raised), threads = workgroup size
- * (multiple of 64 <= 1024, 0 = automatic).  Process-wide.
+ * Tuning / test knobs (process-wide; value 0 restores the automatic choice).  They change
+ * how a launch is cut into workgroups, never its result.  No reference counterpart.
  */
-int msd_set_groupnorm_plan(int split, int threads);
-
-/*
- * Tuning / test knob: bytes each lane of msd_layernorm moves per load (8 or 16;
- * 0 = automatic).  Process-wide.
- */
-int msd_set_layernorm_chunk(int bytes);
-
-/*
- * Tuning / test knob: 16-byte vectors each lane of msd_geglu produces (1, 2 or 4;
- * 0 = automatic).  Process-wide.
- */
-int msd_set_geglu_unroll(int vectors);
+#define MSD_TUNE_GN_SPLIT 0      /* workgroups per (sample, group): power of two <= 64 */
+#define MSD_TUNE_GN_THREADS 1    /* GroupNorm workgroup size: multiple of 64, <= 1024 */
+#define MSD_TUNE_LN_CHUNK 2      /* bytes a LayerNorm lane moves per load: 8 or 16 */
+#define MSD_TUNE_LN_THREADS 3    /* LayerNorm workgroup size: 64, 128, 256 or 512 */
+#define MSD_TUNE_GEGLU_VECTORS 4 /* 16-byte vectors per GEGLU lane: 1, 2 or 4 */
+#define MSD_TUNE_ACT_VECTORS 5   /* 16-byte vectors per lane of SiLU / GELU / quick_GELU: 1, 2 or 4 */
+int msd_set_tuning(int knob, int value);
 
 /*
  * GroupNorm over NCHW, optionally followed by SiLU, in one launch.

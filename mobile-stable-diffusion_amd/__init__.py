@@ -17,11 +17,12 @@ LIB_NN_PATH = os.path.join(CSRC_DIR, "libmsd_nn.so")
 
 DTYPE_F32 = 0
 DTYPE_F16 = 1
+TUNE_GN_SPLIT, TUNE_GN_THREADS, TUNE_LN_CHUNK, TUNE_LN_THREADS, TUNE_GEGLU_VECTORS, TUNE_ACT_VECTORS = range(6)
 
 # every symbol include/msd_hip.h declares
 C_ABI_SYMBOLS = (
     "msd_version", "msd_error_string", "msd_init", "msd_shutdown", "msd_status",
-    "msd_set_groupnorm_plan", "msd_set_layernorm_chunk", "msd_set_geglu_unroll", "msd_groupnorm", "msd_layernorm", "msd_geglu",
+    "msd_set_tuning", "msd_groupnorm", "msd_layernorm", "msd_geglu",
     "msd_silu", "msd_gelu", "msd_quick_gelu", "msd_timestep_embedding", "msd_ddim_timesteps",
 )
 
@@ -50,9 +51,7 @@ def load_library(path=None):
     lib.msd_init.argtypes = [vp]
     lib.msd_shutdown.argtypes = []
     lib.msd_status.argtypes = [vp]
-    lib.msd_set_groupnorm_plan.argtypes = [it, it]
-    lib.msd_set_layernorm_chunk.argtypes = [it]
-    lib.msd_set_geglu_unroll.argtypes = [it]
+    lib.msd_set_tuning.argtypes = [it, it]
     lib.msd_groupnorm.argtypes = [vp, vp, vp, vp, sz, sz, sz, sz, fl, it, it, vp]
     lib.msd_layernorm.argtypes = [vp, vp, vp, vp, sz, sz, fl, it, vp]
     lib.msd_geglu.argtypes = [vp, vp, sz, sz, it, vp]

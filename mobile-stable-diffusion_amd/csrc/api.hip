@@ -63,6 +63,8 @@ hipError_t get_scratch(hipStream_t stream, GnScratch *out) {
     return hipSuccess;
 }
 
+Tuning g_tuning = {0, 0, 0, 0, 0, 0};
+
 }  // namespace msd
 
 using namespace msd;
@@ -117,25 +119,36 @@ int msd_status(void *stream) {
     return flags ? (int)hipErrorLaunchFailure : MSD_OK;
 }
 
-int msd_set_groupnorm_plan(int split, int threads) {
-    if (split < 0 || threads < 0) return MSD_ERR_INVALID_VALUE;
-    if (split > 0 && ((split & (split - 1)) != 0 || split > (int)kGnMaxSplit)) return MSD_ERR_INVALID_VALUE;
-    if (threads > 0 && (threads % 64 != 0 || threads > 1024)) return MSD_ERR_INVALID_VALUE;
-    g_gn_plan_override.split = split;
-    g_gn_plan_override.threads = threads;
-    return MSD_OK;
-}
-
-int msd_set_geglu_unroll(int vectors) {
-    if (vectors != 0 && vectors != 1 && vectors != 2 && vectors != 4) return MSD_ERR_INVALID_VALUE;
-    g_geglu_unroll_override = vectors;
-    return MSD_OK;
-}
-
-int msd_set_layernorm_chunk(int bytes) {
-    if (bytes != 0 && bytes != 8 && bytes != 16) return MSD_ERR_INVALID_VALUE;
-    g_ln_chunk_override = bytes;
-    return MSD_OK;
+int msd_set_tuning(int knob, int value) {
+    if (value < 0) return MSD_ERR_INVALID_VALUE;
+    switch (knob) {
+        case MSD_TUNE_GN_SPLIT:
+            if (value && ((value & (value - 1)) != 0 || value > (int)kGnMaxSplit)) return MSD_ERR_INVALID_VALUE;
+            g_tuning.gn_split = value;
+            return MSD_OK;
+        case MSD_TUNE_GN_THREADS:
+            if (value && (value % 64 != 0 || value > 1024)) return MSD_ERR_INVALID_VALUE;
+            g_tuning.gn_threads = value;
+            return MSD_OK;
+        case MSD_TUNE_LN_CHUNK:
+            if (value && value != 8 && value != 16) return MSD_ERR_INVALID_VALUE;
+            g_tuning.ln_chunk = value;
+            return MSD_OK;
+        case MSD_TUNE_LN_THREADS:
+            if (value && value != 64 && value != 128 && value != 256 && value != 512) return MSD_ERR_INVALID_VALUE;
+            g_tuning.ln_threads = value;
+            return MSD_OK;
+        case MSD_TUNE_GEGLU_VECTORS:
+            if (value && value != 1 && value != 2 && value != 4) return MSD_ERR_INVALID_VALUE;
+            g_tuning.geglu_vectors = value;
+            return MSD_OK;
+        case MSD_TUNE_ACT_VECTORS:
+            if (value && value != 1 && value != 2 && value != 4) return MSD_ERR_INVALID_VALUE;
+            g_tuning.act_vectors = value;
+            return MSD_OK;
+        default:
+            return MSD_ERR_INVALID_VALUE;
+    }
 }
 
 int msd_groupnorm(const void *x, void *y, const float *gamma, const float *beta, size_t batch,

@@ -22,8 +22,6 @@
 
 namespace msd {
 
-GnPlanOverride g_gn_plan_override = {0, 0};
-
 namespace {
 
 constexpr int kGnMaxThreads = 1024;
@@ -301,42 +299,23 @@ struct GnPlan {
     int k;  // 0 = does not fit
 };
 
-// Threads and K for a slice of `vecs` vectors.  Measured on MI355X, workgroups of about
-// 512 lanes finish soonest (enough wavefronts to hide latency, short reduction tail), so
-// among the widths (multiples of 64 in [256, 1024]) that divide the slice into one of the
-// compiled K values the one nearest 512 wins; without an exact fit the tail is masked.
+// Threads and K for a slice of `vecs` vectors.  Measured on MI355X over every UNet shape
+// (workgroups of 256 ... 1024 lanes in steps of 64, 1 - 8 slices per unit): 512 lanes finish
+// soonest whenever the slice is at most 5 vectors per lane, even when the last wavefronts are
+// partly idle (a 320-vector unit: 2.95 us with 512 lanes, 3.18 us with exactly 320); larger
+// slices want 1024 lanes.  The tail of a slice that does not fill K * threads is masked.
 GnPlan plan_slice(uint32_t vecs, uint32_t split, uint32_t force_threads, uint32_t max_k) {
     GnPlan pl{split, 0, 0};
-    if (force_threads) {
+    if (force_threads)
         pl.threads = force_threads;
-        pl.k = round_up_k((vecs + force_threads - 1) / force_threads);
-        if ((uint32_t)pl.k > max_k) pl.k = 0;
-        return pl;
-    }
-    uint32_t best_nt = 0, best_dist = ~0u;
-    for (uint32_t nt = 256; nt <= (uint32_t)kGnMaxThreads; nt += kWave) {
-        if (vecs % nt) continue;
-        const uint32_t k = vecs / nt;
-        if (k > max_k || round_up_k(k) != (int)k) continue;
-        const uint32_t dist = nt > 512 ? nt - 512 : 512 - nt;
-        if (dist < best_dist) {
-            best_dist = dist;
-            best_nt = nt;
-        }
-    }
-    if (best_nt) {
-        pl.threads = best_nt;
-        pl.k = (int)(vecs / best_nt);
-        return pl;
-    }
-    if (vecs > 512u * max_k)
+    else if (vecs > 512u * 5u)
         pl.threads = kGnMaxThreads;
-    else if (vecs >= 512)
+    else if (vecs >= 256)
         pl.threads = 512;
     else
         pl.threads = ((vecs + kWave - 1) / kWave) * kWave;
     pl.k = round_up_k((vecs + pl.threads - 1) / pl.threads);
-    if ((uint32_t)pl.k > max_k) pl.k = 0;
+    if (pl.k == 0 || (uint32_t)pl.k > max_k) pl.k = 0;
     return pl;
 }
 
@@ -388,8 +367,8 @@ int gn_dispatch(const void *xv, void *yv, const float *gamma, const float *beta,
     const bool can_split = units <= kGnMaxUnits;
     if (split > kGnMaxSplit || (split > 1 && !can_split))
         return gn_generic<T>(silu, x, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
-    if (g_gn_plan_override.split > 0) {
-        uint32_t forced = (uint32_t)g_gn_plan_override.split;
+    if (g_tuning.gn_split > 0) {
+        uint32_t forced = (uint32_t)g_tuning.gn_split;
         if (forced > split && can_split && (forced & (forced - 1)) == 0 && forced <= kGnMaxSplit &&
             vec_per_unit >= (size_t)forced * kWave)
             split = forced;
@@ -422,10 +401,10 @@ int gn_dispatch(const void *xv, void *yv, const float *gamma, const float *beta,
         return gn_generic<T>(silu, x, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
 
     uint32_t force_threads = 0;
-    if (g_gn_plan_override.threads >= kWave && g_gn_plan_override.threads <= kGnMaxThreads &&
-        g_gn_plan_override.threads % kWave == 0 &&
-        (size_t)g_gn_plan_override.threads * kMaxK >= p.vec_per_slice)
-        force_threads = (uint32_t)g_gn_plan_override.threads;
+    if (g_tuning.gn_threads >= kWave && g_tuning.gn_threads <= kGnMaxThreads &&
+        g_tuning.gn_threads % kWave == 0 &&
+        (size_t)g_tuning.gn_threads * kMaxK >= p.vec_per_slice)
+        force_threads = (uint32_t)g_tuning.gn_threads;
     const GnPlan pl = plan_slice(p.vec_per_slice, split, force_threads, kMaxK);
     if (pl.k == 0)
         return gn_generic<T>(silu, x, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);

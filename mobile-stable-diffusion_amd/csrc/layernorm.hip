@@ -10,7 +10,9 @@
 namespace msd {
 namespace {
 
-constexpr int kLnThreads = 256;
+constexpr int kLnThreads = 64;      // default workgroup: one wavefront (measured: never slower
+                                    // than 128 / 256 / 512 lanes, 5 - 8 % faster below 1000 rows)
+constexpr int kLnMaxThreads = 512;  // launch bound
 
 // NW dwords (8 or 16 bytes) of T, moved with one instruction.
 template <int NW>
@@ -62,7 +64,7 @@ struct Chunk {
 // covers 64/TL consecutive rows.  Lane (team, j) holds chunks j, j+TL, ... of its row and
 // the gamma / beta of the same columns, all requested before the first use.
 template <typename T, int NW, int VPL, int TL>
-__global__ __launch_bounds__(kLnThreads) void ln_team_kernel(
+__global__ __launch_bounds__(kLnMaxThreads) void ln_team_kernel(
     const T *x, T *y, const float *__restrict__ gamma, const float *__restrict__ beta,
     uint32_t rows, float eps, float inv_dim) {
     typedef Chunk<T, NW> C;
@@ -70,7 +72,7 @@ __global__ __launch_bounds__(kLnThreads) void ln_team_kernel(
     constexpr int N = C::N;
     constexpr int RPW = kWave / TL;  // rows per wavefront
     const uint32_t lane = threadIdx.x & (kWave - 1);
-    const uint32_t wave = blockIdx.x * (kLnThreads / kWave) + threadIdx.x / kWave;
+    const uint32_t wave = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
     const uint32_t row = wave * RPW + lane / TL;
     const uint32_t j = lane % TL;
     const bool live = row < rows;
@@ -163,10 +165,11 @@ __global__ __launch_bounds__(kLnThreads) void ln_generic_kernel(
 template <typename T, int NW, int VPL, int TL>
 void ln_launch(const T *x, T *y, const float *gamma, const float *beta, uint32_t rows, float eps,
                float inv_dim, hipStream_t stream) {
-    constexpr uint32_t rows_per_block = (kWave / TL) * (kLnThreads / kWave);
+    const uint32_t threads = g_tuning.ln_threads ? (uint32_t)g_tuning.ln_threads : (uint32_t)kLnThreads;
+    const uint32_t rows_per_block = (kWave / TL) * (threads / kWave);
     const uint32_t blocks = (rows + rows_per_block - 1) / rows_per_block;
-    hipLaunchKernelGGL((ln_team_kernel<T, NW, VPL, TL>), dim3(blocks), dim3(kLnThreads), 0, stream, x,
-                       y, gamma, beta, rows, eps, inv_dim);
+    hipLaunchKernelGGL((ln_team_kernel<T, NW, VPL, TL>), dim3(blocks), dim3(threads), 0, stream, x, y,
+                       gamma, beta, rows, eps, inv_dim);
 }
 
 template <typename T, int NW, int TL>
@@ -207,8 +210,6 @@ bool ln_try(const T *x, T *y, const float *gamma, const float *beta, uint32_t ro
 
 }  // namespace
 
-int g_ln_chunk_override = 0;  // 0 = automatic, 8 or 16 = forced chunk bytes (tuning)
-
 template <typename T>
 int ln_dispatch(const void *xv, void *yv, const float *gamma, const float *beta, size_t rows,
                 size_t dim, float eps, hipStream_t stream) {
@@ -232,8 +233,8 @@ int ln_dispatch(const void *xv, void *yv, const float *gamma, const float *beta,
             while ((d / n16) % tl != 0) tl /= 2;
             prefer8 = tl < kWave && (d / tl) > 16;
         }
-        if (g_ln_chunk_override == 8) prefer8 = true;
-        if (g_ln_chunk_override == 16) prefer8 = false;
+        if (g_tuning.ln_chunk == 8) prefer8 = true;
+        if (g_tuning.ln_chunk == 16) prefer8 = false;
         if (prefer8) done = ln_try<T, 2>(x, y, gamma, beta, r, d, eps, inv_dim, stream);
         if (!done) done = ln_try<T, 4>(x, y, gamma, beta, r, d, eps, inv_dim, stream);
         if (!done && !prefer8) done = ln_try<T, 2>(x, y, gamma, beta, r, d, eps, inv_dim, stream);

@@ -27,14 +27,16 @@ struct GnScratch {
 // Per-(device, stream) scratch, created on first use (hipMalloc + hipMemset).
 hipError_t get_scratch(hipStream_t stream, GnScratch *out);
 
-// Forced launch plan for msd_groupnorm (0 = choose automatically).
-struct GnPlanOverride {
-    int split;
-    int threads;
+// Tuning overrides set through msd_set_tuning (0 = choose automatically).
+struct Tuning {
+    int gn_split;
+    int gn_threads;
+    int ln_chunk;
+    int ln_threads;
+    int geglu_vectors;
+    int act_vectors;
 };
-extern GnPlanOverride g_gn_plan_override;
-extern int g_geglu_unroll_override;  // 0 = automatic, 1 / 2 / 4 = forced vectors per lane
-extern int g_ln_chunk_override;  // 0 = automatic, 8 / 16 = forced LayerNorm chunk bytes
+extern Tuning g_tuning;
 
 // ---- per-dtype dispatchers (T = float or __half), defined in the kernel files ----
 template <typename T>

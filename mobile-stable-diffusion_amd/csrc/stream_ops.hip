@@ -75,11 +75,10 @@ __global__ __launch_bounds__(kStreamThreads) void geglu_generic_kernel(
 
 // y[i] = OP(x[i]); y may alias x: a lane reads its vectors before it writes them,
 // and in the ragged last block the duplicated reads are never written back.
-template <typename T, typename OP>
+template <typename T, typename OP, int U>
 __global__ __launch_bounds__(kStreamThreads) void act_kernel(const T *x, T *y, uint32_t vecs,
                                                              size_t n) {
     constexpr int EPV = Store<T>::EPV;
-    constexpr int U = kStreamUnroll;
     const u32x4 *in = reinterpret_cast<const u32x4 *>(x);
     u32x4 *o = reinterpret_cast<u32x4 *>(y);
     const uint32_t block_base = blockIdx.x * (kStreamThreads * U);
@@ -143,14 +142,12 @@ __global__ __launch_bounds__(256) void timestep_embedding_kernel(
 }
 
 // ---- streaming dispatch ----------------------------------------------------
-inline uint32_t stream_blocks(size_t vecs) {
-    const size_t per_block = (size_t)kStreamThreads * kStreamUnroll;
+inline uint32_t stream_blocks(size_t vecs, int unroll) {
+    const size_t per_block = (size_t)kStreamThreads * unroll;
     return (uint32_t)((vecs + per_block - 1) / per_block);
 }
 
 }  // namespace
-
-int g_geglu_unroll_override = 0;  // 0 = automatic; 1, 2 or 4 vectors per lane (tuning)
 
 template <typename T>
 int geglu_dispatch(const void *pv, void *ov, size_t rows, size_t inner, hipStream_t stream) {
@@ -165,7 +162,7 @@ int geglu_dispatch(const void *pv, void *ov, size_t rows, size_t inner, hipStrea
         // one vector per lane: these launches are short enough that a lane's dependent ALU chain
         // is on the critical path, and more, lighter wavefronts overlap it with other loads
         // (measured 9 - 30 % faster than 4 vectors per lane at every UNet shape)
-        const int unroll = g_geglu_unroll_override ? g_geglu_unroll_override : 1;
+        const int unroll = g_tuning.geglu_vectors ? g_tuning.geglu_vectors : 1;
         const uint32_t ov = (uint32_t)out_vecs;
         auto blocks = [&](int u) { return (uint32_t)((out_vecs + kStreamThreads * u - 1) / (kStreamThreads * u)); };
         if (unroll == 1)
@@ -193,9 +190,17 @@ int act_launch(const void *xv, void *yv, size_t n, hipStream_t stream) {
     if (n == 0) return MSD_OK;
     const size_t vecs = n / EPV;
     if (aligned16(x) && aligned16(y) && vecs < 0x7FFFFFFFull) {
-        const uint32_t blocks = vecs ? stream_blocks(vecs) : 1u;
-        hipLaunchKernelGGL((act_kernel<T, OP>), dim3(blocks), dim3(kStreamThreads), 0, stream, x, y,
-                           (uint32_t)vecs, n);
+        const int unroll = g_tuning.act_vectors ? g_tuning.act_vectors : kStreamUnroll;
+        const uint32_t blocks = vecs ? stream_blocks(vecs, unroll) : 1u;
+        if (unroll == 4)
+            hipLaunchKernelGGL((act_kernel<T, OP, 4>), dim3(blocks), dim3(kStreamThreads), 0, stream, x, y,
+                               (uint32_t)vecs, n);
+        else if (unroll == 2)
+            hipLaunchKernelGGL((act_kernel<T, OP, 2>), dim3(blocks), dim3(kStreamThreads), 0, stream, x, y,
+                               (uint32_t)vecs, n);
+        else
+            hipLaunchKernelGGL((act_kernel<T, OP, 1>), dim3(blocks), dim3(kStreamThreads), 0, stream, x, y,
+                               (uint32_t)vecs, n);
     } else {
         const size_t want = (n + kStreamThreads - 1) / kStreamThreads;
         hipLaunchKernelGGL((act_generic_kernel<T, OP>),

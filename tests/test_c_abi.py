@@ -19,7 +19,7 @@ def _declared_symbols():
 def test_header_symbols_are_exported(msd):
     lib = msd.load_library()
     declared = _declared_symbols()
-    assert len(declared) >= 14
+    assert len(declared) >= 13
     for name in declared:
         assert hasattr(lib, name), "libmsd_hip.so does not export %s" % name
     assert sorted(msd.C_ABI_SYMBOLS) == declared  # the ctypes table covers the whole header
@@ -69,9 +69,11 @@ def test_argument_validation_needs_no_gpu(msd):
     assert lib.msd_geglu(None, None, 4, 64, 0, None) == 1
     assert lib.msd_silu(None, None, 4, 0, None) == 1
     assert lib.msd_timestep_embedding(None, None, 2, 321, 10000.0, 0, None) == 1
-    assert lib.msd_set_groupnorm_plan(3, 0) == 1
-    assert lib.msd_set_groupnorm_plan(0, 100) == 1
-    assert lib.msd_set_groupnorm_plan(0, 0) == 0
+    assert lib.msd_set_tuning(0, 3) == 1      # split must be a power of two
+    assert lib.msd_set_tuning(1, 100) == 1    # threads must be a multiple of 64
+    assert lib.msd_set_tuning(2, 12) == 1 and lib.msd_set_tuning(4, 3) == 1 and lib.msd_set_tuning(99, 1) == 1
+    for knob in range(6):
+        assert lib.msd_set_tuning(knob, 0) == 0
 
 
 def test_missing_library_fails_loudly(msd):

@@ -97,12 +97,14 @@ def test_groupnorm_every_split_factor(msd, orc, cuda, split, threads):
     x = orc.normal((2, 320, 64, 64), seed=88, sigma=2.0, mean=1.0)
     g, b = _affine(orc, 320, 88)
     try:
-        assert lib.msd_set_groupnorm_plan(split, threads) == 0
+        assert lib.msd_set_tuning(msd.TUNE_GN_SPLIT, split) == 0
+        assert lib.msd_set_tuning(msd.TUNE_GN_THREADS, threads) == 0
         for half in (False, True):
             _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half)
             _run_groupnorm(msd, orc, cuda, x[:1, :96, :24, :24].copy(), g[:96], b[:96], 32, 1e-5, True, half)
     finally:
-        lib.msd_set_groupnorm_plan(0, 0)
+        lib.msd_set_tuning(msd.TUNE_GN_SPLIT, 0)
+        lib.msd_set_tuning(msd.TUNE_GN_THREADS, 0)
     assert msd.status() == 0
 
 
@@ -113,12 +115,12 @@ def test_groupnorm_repeated_launches_reuse_scratch(msd, orc, cuda):
     try:
         for rep in range(3):
             for i, shp in enumerate(shapes):
-                lib.msd_set_groupnorm_plan([4, 2, 8, 1][(rep + i) % 4], 0)
+                lib.msd_set_tuning(msd.TUNE_GN_SPLIT, [4, 2, 8, 1][(rep + i) % 4])
                 x = orc.normal(shp, seed=900 + i + 10 * rep, sigma=2.0)
                 g, b = _affine(orc, shp[1], 900 + i)
                 _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half=True)
     finally:
-        lib.msd_set_groupnorm_plan(0, 0)
+        lib.msd_set_tuning(msd.TUNE_GN_SPLIT, 0)
     assert msd.status() == 0
 
 
@@ -225,11 +227,12 @@ def test_layernorm_dims_and_ragged_rows(msd, orc, cuda, rows, dim, half):
         assert_close_f32(got, ref, what="ln dims f32")
 
 
-@pytest.mark.parametrize("chunk", [8, 16])
-def test_layernorm_forced_chunk_width(msd, orc, cuda, chunk):
+@pytest.mark.parametrize("chunk,threads", [(8, 0), (16, 0), (8, 64), (16, 512), (0, 128)])
+def test_layernorm_forced_chunk_width(msd, orc, cuda, chunk, threads):
     lib = msd.load_library()
     try:
-        assert lib.msd_set_layernorm_chunk(chunk) == 0
+        assert lib.msd_set_tuning(msd.TUNE_LN_CHUNK, chunk) == 0
+        assert lib.msd_set_tuning(msd.TUNE_LN_THREADS, threads) == 0
         for rows, dim, half in [(8192, 320, True), (300, 640, True), (77, 768, False), (33, 1280, False),
                                 (5, 64, True), (5, 64, False), (9, 2048, True)]:
             x = orc.normal((rows, dim), seed=rows + dim + chunk, sigma=1.5, mean=-1.0)
@@ -242,7 +245,8 @@ def test_layernorm_forced_chunk_width(msd, orc, cuda, chunk):
             else:
                 assert_close_f32(got, ref, what="ln chunk f32")
     finally:
-        lib.msd_set_layernorm_chunk(0)
+        lib.msd_set_tuning(msd.TUNE_LN_CHUNK, 0)
+        lib.msd_set_tuning(msd.TUNE_LN_THREADS, 0)
 
 
 def test_layernorm_in_place_fixtures_and_empty(msd, orc, golden, cuda):
@@ -284,13 +288,17 @@ def test_geglu_shapes_fp32_fp16(msd, orc, golden, cuda, rows, inner, half):
 def test_geglu_forced_vectors_per_lane(msd, orc, cuda, unroll):
     lib = msd.load_library()
     try:
-        assert lib.msd_set_geglu_unroll(unroll) == 0
+        assert lib.msd_set_tuning(msd.TUNE_GEGLU_VECTORS, unroll) == 0
+        assert lib.msd_set_tuning(msd.TUNE_ACT_VECTORS, unroll) == 0
+        x = orc.normal((3, 1031), seed=unroll, sigma=3.0)
+        assert_close_f32(msd.silu(_to_dev(x, cuda)).cpu().numpy(), orc.silu(x), what="silu unroll")
         for rows, inner in [(2048, 2560), (77, 1288), (3, 8), (1000, 24)]:
             proj = orc.round_to_half(orc.normal((rows, 2 * inner), seed=rows + unroll, sigma=1.5))
             got = msd.geglu(_to_dev(proj, cuda, True)).float().cpu().numpy()
             assert_close_f16(got, orc.round_to_half(orc.geglu(proj)), "geglu unroll")
     finally:
-        lib.msd_set_geglu_unroll(0)
+        lib.msd_set_tuning(msd.TUNE_GEGLU_VECTORS, 0)
+        lib.msd_set_tuning(msd.TUNE_ACT_VECTORS, 0)
 
 
 @pytest.mark.parametrize("name", ["silu", "gelu", "quick_gelu"])
