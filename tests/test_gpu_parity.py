@@ -365,3 +365,108 @@ def test_config5_timesteps_feed_embedding_bit_exact_integers(msd, orc, cuda):
     rnd = orc.uniform_int(2, 5001, 0, 999)
     emb2 = msd.timestep_embedding(torch.from_numpy(rnd).to(cuda), 320, dtype=torch.float16)
     assert emb2.shape == (2, 320)
+
+
+# ----------------------------------------------------------------- launch machinery
+def test_groupnorm_graph_replay_matches_eager(msd, orc, cuda):
+    """The cross-workgroup exchange keeps per-unit launch counts in device memory, so a
+    captured graph must give on every replay what the eager launch gives."""
+    torch = _torch()
+    stream = torch.cuda.Stream()
+    shapes = [(2, 320, 4096), (2, 960, 1024), (2, 1280, 64), (2, 640, 4096)]
+    xs0 = [orc.round_to_half(orc.normal(s, seed=700 + i, sigma=2.0)) for i, s in enumerate(shapes)]
+    gbs = [_affine(orc, s[1], 700 + i) for i, s in enumerate(shapes)]
+    with torch.cuda.stream(stream):
+        msd.init()
+        xs = [_to_dev(x, cuda, True) for x in xs0]
+        ys = [torch.empty_like(x) for x in xs]
+        zs = [x.clone() for x in xs]
+        gd = [(_to_dev(g, cuda), _to_dev(b, cuda)) for g, b in gbs]
+
+        def body():
+            for x, y, z, (g, b) in zip(xs, ys, zs, gd):
+                msd.groupnorm(x, g, b, 32, 1e-5, True, out=y)   # out of place
+                msd.groupnorm(z, g, b, 32, 1e-6, False, out=z)  # in place
+        body()
+        torch.cuda.synchronize()
+        eager = [(y.clone(), z.clone()) for y, z in zip(ys, zs)]
+        for x, z in zip(xs, zs):
+            z.copy_(x)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            body()
+        for rep in range(5):
+            for x, y, z in zip(xs, ys, zs):  # eager work between replays
+                y.zero_()
+                z.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            for y, z, (ey, ez) in zip(ys, zs, eager):
+                assert torch.equal(y, ey) and torch.equal(z, ez), "replay %d differs from the eager result" % rep
+        assert msd.status() == 0
+    # and the eager result is the right one
+    for x0, (g, b), (ey, ez) in zip(xs0, gbs, eager):
+        assert_close_f16(ey.float().cpu().numpy(), orc.round_to_half(orc.groupnorm(x0, g, b, 32, 1e-5, True)), "gn graph")
+        assert_close_f16(ez.float().cpu().numpy(), orc.round_to_half(orc.groupnorm(x0, g, b, 32, 1e-6, False)), "gn graph")
+
+
+def test_groupnorm_two_streams_have_private_scratch(msd, orc, cuda):
+    torch = _torch()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    x1 = orc.round_to_half(orc.normal((2, 640, 4096), seed=801, sigma=2.0))
+    x2 = orc.round_to_half(orc.normal((2, 960, 4096), seed=802, sigma=1.0, mean=3.0))
+    g1, b1 = _affine(orc, 640, 801)
+    g2, b2 = _affine(orc, 960, 802)
+    d1, d2 = _to_dev(x1, cuda, True), _to_dev(x2, cuda, True)
+    a1 = (_to_dev(g1, cuda), _to_dev(b1, cuda))
+    a2 = (_to_dev(g2, cuda), _to_dev(b2, cuda))
+    torch.cuda.synchronize()
+    outs1, outs2 = [], []
+    for _ in range(20):  # interleaved submissions keep both streams busy at once
+        with torch.cuda.stream(s1):
+            outs1.append(msd.groupnorm(d1, *a1, 32, 1e-5, True))
+        with torch.cuda.stream(s2):
+            outs2.append(msd.groupnorm(d2, *a2, 32, 1e-5, True))
+    torch.cuda.synchronize()
+    r1 = orc.round_to_half(orc.groupnorm(x1, g1, b1, 32, 1e-5, True))
+    r2 = orc.round_to_half(orc.groupnorm(x2, g2, b2, 32, 1e-5, True))
+    for o in outs1:
+        assert torch.equal(o, outs1[0])
+    for o in outs2:
+        assert torch.equal(o, outs2[0])
+    assert_close_f16(outs1[0].float().cpu().numpy(), r1, "stream 1")
+    assert_close_f16(outs2[0].float().cpu().numpy(), r2, "stream 2")
+    lib = msd.load_library()
+    import ctypes
+    assert lib.msd_status(ctypes.c_void_p(s1.cuda_stream)) == 0
+    assert lib.msd_status(ctypes.c_void_p(s2.cuda_stream)) == 0
+
+
+def test_groupnorm_many_units_and_register_limits(msd, orc, cuda):
+    # more units than scratch slots (never split), and float units that need a split to fit
+    for shape, groups, half in [((300, 64, 4, 8), 32, True),     # 9600 units
+                                ((1, 32, 64, 64), 2, False),     # 65536-element float units
+                                ((2, 8, 128, 128), 1, False),    # 131072-element float units
+                                ((1, 16, 256, 256), 1, True)]:   # 1 Mi-element half unit: 64 slices
+        x = orc.normal(shape, seed=sum(shape), sigma=1.7, mean=-0.3)
+        xin = orc.round_to_half(x) if half else x
+        g, b = _affine(orc, shape[1], 41)
+        ref = orc.groupnorm64(xin, g, b, groups, 1e-5, True)
+        got = msd.groupnorm(_to_dev(xin, cuda, half), _to_dev(g, cuda), _to_dev(b, cuda), groups, 1e-5, True)
+        got = got.float().cpu().numpy()
+        if half:
+            assert_close_f16(got, orc.round_to_half(ref.astype(np.float32)), "gn limits f16")
+        else:
+            assert_close_f32(got, ref, what="gn limits f32")
+    assert msd.status() == 0
+
+
+def test_shutdown_then_reuse(msd, orc, cuda):
+    lib = msd.load_library()
+    x = orc.normal((2, 320, 4096), seed=5, sigma=2.0)
+    g, b = _affine(orc, 320, 5)
+    _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half=True)
+    _torch().cuda.synchronize()
+    assert lib.msd_shutdown() == 0
+    _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half=True)  # scratch is created again
+    assert msd.status() == 0
