@@ -89,6 +89,34 @@ int msd_layernorm(const void *x, void *y, const float *gamma, const float *beta,
                   size_t dim, float eps, int dtype, void *stream);
 
 /*
+ * The two additions the reference runs right before its norms, and their fusions.
+ *   msd_elemwise_add   c[i] = a[i] + b[i]                 K/util.cl:1-12 (the residual adds
+ *                      of M/nn/BasicTransformerBlock.cpp:126-134,149-156,170-177)
+ *   msd_chunkwise_add  c[i] = a[i] + chunk[i / chunk_size] K/util.cl:136-148 (the time-embedding
+ *                      add of M/nn/ResBlock.cpp:188-199; chunk holds one value per run of
+ *                      chunk_size elements, i.e. [batch, channels] with chunk_size = hw)
+ * c may alias a (every reference call site does) or b.
+ *
+ *   msd_chunk_add_groupnorm  = msd_chunkwise_add(x, chunk, tmp, ., hw) followed by
+ *                      msd_groupnorm(tmp, y, ...), bit for bit, without the pass over tmp:
+ *                      replaces M/nn/ResBlock.cpp:188-199 + 222-232 in one launch.
+ *                      chunk is [batch, channels] in the activation storage type.
+ *   msd_add_layernorm  = msd_elemwise_add(a, b, sum) followed by msd_layernorm(sum, y, ...), bit
+ *                      for bit, in one launch; `sum` is written because the reference keeps it
+ *                      as the next residual (M/nn/BasicTransformerBlock.cpp:126-136,149-158).
+ *                      sum may alias a or b.
+ */
+int msd_elemwise_add(const void *a, const void *b, void *c, size_t n, int dtype, void *stream);
+int msd_chunkwise_add(const void *a, const void *chunk, void *c, size_t n, size_t chunk_size,
+                      int dtype, void *stream);
+int msd_chunk_add_groupnorm(const void *x, const void *chunk, void *y, const float *gamma,
+                            const float *beta, size_t batch, size_t channels, size_t hw,
+                            size_t groups, float eps, int fuse_silu, int dtype, void *stream);
+int msd_add_layernorm(const void *a, const void *b, void *sum, void *y, const float *gamma,
+                      const float *beta, size_t rows, size_t dim, float eps, int dtype,
+                      void *stream);
+
+/*
  * GEGLU epilogue on an already projected tensor: proj is [rows, 2*inner] with
  * the value in the first half of each row and the gate in the second;
  * out[r, c] = proj[r, c] * gelu_erf(proj[r, inner + c]).  Replaces the

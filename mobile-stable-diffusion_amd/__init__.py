@@ -24,6 +24,7 @@ C_ABI_SYMBOLS = (
     "msd_version", "msd_error_string", "msd_init", "msd_shutdown", "msd_status",
     "msd_set_tuning", "msd_groupnorm", "msd_layernorm", "msd_geglu",
     "msd_silu", "msd_gelu", "msd_quick_gelu", "msd_timestep_embedding", "msd_ddim_timesteps",
+    "msd_elemwise_add", "msd_chunkwise_add", "msd_chunk_add_groupnorm", "msd_add_layernorm",
 )
 
 _lib = None
@@ -55,6 +56,10 @@ def load_library(path=None):
     lib.msd_groupnorm.argtypes = [vp, vp, vp, vp, sz, sz, sz, sz, fl, it, it, vp]
     lib.msd_layernorm.argtypes = [vp, vp, vp, vp, sz, sz, fl, it, vp]
     lib.msd_geglu.argtypes = [vp, vp, sz, sz, it, vp]
+    lib.msd_elemwise_add.argtypes = [vp, vp, vp, sz, it, vp]
+    lib.msd_chunkwise_add.argtypes = [vp, vp, vp, sz, sz, it, vp]
+    lib.msd_chunk_add_groupnorm.argtypes = [vp, vp, vp, vp, vp, sz, sz, sz, sz, fl, it, it, vp]
+    lib.msd_add_layernorm.argtypes = [vp, vp, vp, vp, vp, vp, sz, sz, fl, it, vp]
     for name in ("msd_silu", "msd_gelu", "msd_quick_gelu"):
         getattr(lib, name).argtypes = [vp, vp, sz, it, vp]
     lib.msd_timestep_embedding.argtypes = [vp, vp, sz, sz, fl, it, vp]
@@ -108,6 +113,45 @@ def groupnorm(x, gamma, beta, groups, eps=1e-5, fuse_silu=False, out=None):
     hw = x.numel() // (batch * channels) if batch * channels else 0
     check(load_library().msd_groupnorm(_dev(x), _dev(out), _dev(gamma), _dev(beta), batch, channels,
                                        hw, groups, eps, int(fuse_silu), _dtype_code(x), _stream()))
+    return out
+
+
+def chunk_add_groupnorm(x, chunk, gamma, beta, groups, eps=1e-5, fuse_silu=False, out=None):
+    """GroupNorm(x + chunk[:, :, None]) (+ SiLU); chunk: [batch, C] in x's dtype."""
+    import torch
+    out = torch.empty_like(x) if out is None else out
+    batch, channels = x.shape[0], x.shape[1]
+    hw = x.numel() // (batch * channels) if batch * channels else 0
+    check(load_library().msd_chunk_add_groupnorm(_dev(x), _dev(chunk), _dev(out), _dev(gamma), _dev(beta),
+                                                 batch, channels, hw, groups, eps, int(fuse_silu),
+                                                 _dtype_code(x), _stream()))
+    return out
+
+
+def add_layernorm(a, b, gamma, beta, eps=1e-5, sum_out=None, out=None):
+    """Returns (a + b, LayerNorm(a + b)); sum_out may be a or b."""
+    import torch
+    sum_out = torch.empty_like(a) if sum_out is None else sum_out
+    out = torch.empty_like(a) if out is None else out
+    dim = a.shape[-1]
+    rows = a.numel() // dim if dim else 0
+    check(load_library().msd_add_layernorm(_dev(a), _dev(b), _dev(sum_out), _dev(out), _dev(gamma),
+                                           _dev(beta), rows, dim, eps, _dtype_code(a), _stream()))
+    return sum_out, out
+
+
+def elemwise_add(a, b, out=None):
+    import torch
+    out = torch.empty_like(a) if out is None else out
+    check(load_library().msd_elemwise_add(_dev(a), _dev(b), _dev(out), a.numel(), _dtype_code(a), _stream()))
+    return out
+
+
+def chunkwise_add(a, chunk, chunk_size, out=None):
+    import torch
+    out = torch.empty_like(a) if out is None else out
+    check(load_library().msd_chunkwise_add(_dev(a), _dev(chunk), _dev(out), a.numel(), chunk_size,
+                                           _dtype_code(a), _stream()))
     return out
 
 
@@ -201,11 +245,13 @@ def load_nn_library(path=None):
         "msdnn_groupnorm_init": (it, [vp]),
         "msdnn_groupnorm_check": (it, [vp, sz, it]),
         "msdnn_groupnorm_forward": (it, [vp, vp, vp, sz, it]),
+        "msdnn_groupnorm_forward_chunk": (it, [vp, vp, vp, sz, vp, sz, it]),
         "msdnn_groupnorm_destroy": (None, [vp]),
         "msdnn_layernorm_create": (vp, [vp, sz, cp, cp, fl]),
         "msdnn_layernorm_init": (it, [vp]),
         "msdnn_layernorm_check": (it, [vp, sz, it]),
         "msdnn_layernorm_forward": (it, [vp, vp, vp, sz, it]),
+        "msdnn_layernorm_forward_add": (it, [vp, vp, vp, vp, vp, sz, it]),
         "msdnn_layernorm_destroy": (None, [vp]),
         "msdnn_geglu_create": (vp, [vp, sz, sz]),
         "msdnn_geglu_weight_shape": (it, [vp, szp, szp]),

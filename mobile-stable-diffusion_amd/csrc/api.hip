@@ -151,27 +151,74 @@ int msd_set_tuning(int knob, int value) {
     }
 }
 
-int msd_groupnorm(const void *x, void *y, const float *gamma, const float *beta, size_t batch,
-                  size_t channels, size_t hw, size_t groups, float eps, int fuse_silu, int dtype,
-                  void *stream) {
+static int groupnorm_entry(const void *x, const void *chunk, void *y, const float *gamma,
+                           const float *beta, size_t batch, size_t channels, size_t hw, size_t groups,
+                           float eps, int fuse_silu, int dtype, void *stream) {
     if (groups == 0 || channels == 0 || channels % groups != 0) return MSD_ERR_INVALID_VALUE;
     if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
     if (batch * hw != 0 && (!x || !y || !gamma || !beta)) return MSD_ERR_INVALID_VALUE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == MSD_DTYPE_F32)
-        return gn_dispatch<float>(x, y, gamma, beta, batch, channels, hw, groups, eps,
+        return gn_dispatch<float>(x, chunk, y, gamma, beta, batch, channels, hw, groups, eps,
                                   fuse_silu != 0, s);
-    return gn_dispatch<__half>(x, y, gamma, beta, batch, channels, hw, groups, eps, fuse_silu != 0,
-                               s);
+    return gn_dispatch<__half>(x, chunk, y, gamma, beta, batch, channels, hw, groups, eps,
+                               fuse_silu != 0, s);
+}
+
+int msd_groupnorm(const void *x, void *y, const float *gamma, const float *beta, size_t batch,
+                  size_t channels, size_t hw, size_t groups, float eps, int fuse_silu, int dtype,
+                  void *stream) {
+    return groupnorm_entry(x, nullptr, y, gamma, beta, batch, channels, hw, groups, eps, fuse_silu,
+                           dtype, stream);
+}
+
+int msd_chunk_add_groupnorm(const void *x, const void *chunk, void *y, const float *gamma,
+                            const float *beta, size_t batch, size_t channels, size_t hw,
+                            size_t groups, float eps, int fuse_silu, int dtype, void *stream) {
+    if (batch * hw != 0 && !chunk) return MSD_ERR_INVALID_VALUE;
+    return groupnorm_entry(x, chunk, y, gamma, beta, batch, channels, hw, groups, eps, fuse_silu,
+                           dtype, stream);
+}
+
+static int layernorm_entry(const void *x, const void *res, void *sum, void *y, const float *gamma,
+                           const float *beta, size_t rows, size_t dim, float eps, int dtype,
+                           void *stream) {
+    if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
+    if (rows * dim != 0 && (!x || !y || !gamma || !beta)) return MSD_ERR_INVALID_VALUE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == MSD_DTYPE_F32)
+        return ln_dispatch<float>(x, res, sum, y, gamma, beta, rows, dim, eps, s);
+    return ln_dispatch<__half>(x, res, sum, y, gamma, beta, rows, dim, eps, s);
 }
 
 int msd_layernorm(const void *x, void *y, const float *gamma, const float *beta, size_t rows,
                   size_t dim, float eps, int dtype, void *stream) {
+    return layernorm_entry(x, nullptr, nullptr, y, gamma, beta, rows, dim, eps, dtype, stream);
+}
+
+int msd_add_layernorm(const void *a, const void *b, void *sum, void *y, const float *gamma,
+                      const float *beta, size_t rows, size_t dim, float eps, int dtype,
+                      void *stream) {
+    if (rows * dim != 0 && (!b || !sum)) return MSD_ERR_INVALID_VALUE;
+    return layernorm_entry(a, b, sum, y, gamma, beta, rows, dim, eps, dtype, stream);
+}
+
+int msd_elemwise_add(const void *a, const void *b, void *c, size_t n, int dtype, void *stream) {
     if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
-    if (rows * dim != 0 && (!x || !y || !gamma || !beta)) return MSD_ERR_INVALID_VALUE;
+    if (n != 0 && (!a || !b || !c)) return MSD_ERR_INVALID_VALUE;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dtype == MSD_DTYPE_F32) return ln_dispatch<float>(x, y, gamma, beta, rows, dim, eps, s);
-    return ln_dispatch<__half>(x, y, gamma, beta, rows, dim, eps, s);
+    if (dtype == MSD_DTYPE_F32) return add_dispatch<float>(a, b, c, n, 0, s);
+    return add_dispatch<__half>(a, b, c, n, 0, s);
+}
+
+int msd_chunkwise_add(const void *a, const void *chunk, void *c, size_t n, size_t chunk_size,
+                      int dtype, void *stream) {
+    if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
+    if (chunk_size == 0) return MSD_ERR_INVALID_VALUE;
+    if (n != 0 && (!a || !chunk || !c)) return MSD_ERR_INVALID_VALUE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == MSD_DTYPE_F32) return add_dispatch<float>(a, chunk, c, n, chunk_size, s);
+    return add_dispatch<__half>(a, chunk, c, n, chunk_size, s);
 }
 
 int msd_geglu(const void *proj, void *out, size_t rows, size_t inner, int dtype, void *stream) {

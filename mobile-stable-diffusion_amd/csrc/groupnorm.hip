@@ -58,7 +58,8 @@ __device__ __forceinline__ unsigned long long tagged(uint32_t tag, float v) {
 
 // FULL: every lane owns exactly K vectors (no masking anywhere).
 template <typename T, int K, bool SILU, bool FULL>
-__device__ __forceinline__ void gn_body(const T *x, T *y, const float *__restrict__ gamma,
+__device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
+                                        const float *__restrict__ gamma,
                                         const float *__restrict__ beta, const GnScratch &scratch,
                                         const GnParams &p, uint32_t unit, uint32_t slice,
                                         uint32_t v_begin, uint32_t v_end, float *red_a,
@@ -84,10 +85,25 @@ __device__ __forceinline__ void gn_body(const T *x, T *y, const float *__restric
         vidx[k] = FULL ? v : min(v, v_end - 1);
         raw[k] = load_stream(xin + vidx[k]);
     }
+    const uint32_t ch0 = (unit % p.groups) * p.ch_per_group;
+    // optional per-(sample, channel) addend applied before the statistics (the reference's
+    // chunkwise_add pass): the sum replaces the slice in registers, rounded to the storage
+    // type exactly as a separate add kernel would have stored it
+    if (chunk != nullptr) {  // uniform
+        const T *cb = chunk + (size_t)(unit / p.groups) * (p.groups * p.ch_per_group);
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            const float cv = Store<T>::load1(cb + ch0 + fast_div(vidx[k], p.hw_vec));
+            float f[EPV];
+            Store<T>::unpack(raw[k], f);
+#pragma unroll
+            for (int e = 0; e < EPV; e++) f[e] += cv;
+            raw[k] = Store<T>::pack(f);
+        }
+    }
     // per-vector channel affine: fetched up front while the data is in flight when the
     // registers allow it, otherwise just before use
     constexpr bool kPrefetchAffine = K <= 6;
-    const uint32_t ch0 = (unit % p.groups) * p.ch_per_group;
     float ga[kPrefetchAffine ? K : 1], be[kPrefetchAffine ? K : 1];
     if (kPrefetchAffine) {
 #pragma unroll
@@ -227,8 +243,8 @@ __device__ __forceinline__ void gn_body(const T *x, T *y, const float *__restric
 
 template <typename T, int K, bool SILU>
 __global__ __launch_bounds__(kGnMaxThreads) void gn_slice_kernel(
-    const T *x, T *y, const float *__restrict__ gamma, const float *__restrict__ beta,
-    GnScratch scratch, GnParams p) {
+    const T *x, const T *chunk, T *y, const float *__restrict__ gamma,
+    const float *__restrict__ beta, GnScratch scratch, GnParams p) {
     __shared__ float red_a[kGnMaxThreads / kWave];
     __shared__ float red_b[kGnMaxThreads / kWave];
     __shared__ float stats[2];
@@ -237,10 +253,10 @@ __global__ __launch_bounds__(kGnMaxThreads) void gn_slice_kernel(
     const uint32_t v_begin = slice * p.vec_per_slice;
     const uint32_t v_end = min(p.vec_per_unit, v_begin + p.vec_per_slice);
     if (v_end - v_begin == K * blockDim.x)  // uniform over the workgroup
-        gn_body<T, K, SILU, true>(x, y, gamma, beta, scratch, p, unit, slice, v_begin, v_end, red_a,
-                                  red_b, stats);
+        gn_body<T, K, SILU, true>(x, chunk, y, gamma, beta, scratch, p, unit, slice, v_begin, v_end,
+                                  red_a, red_b, stats);
     else
-        gn_body<T, K, SILU, false>(x, y, gamma, beta, scratch, p, unit, slice, v_begin, v_end,
+        gn_body<T, K, SILU, false>(x, chunk, y, gamma, beta, scratch, p, unit, slice, v_begin, v_end,
                                    red_a, red_b, stats);
 }
 
@@ -248,26 +264,35 @@ __global__ __launch_bounds__(kGnMaxThreads) void gn_slice_kernel(
 // scalar accesses (the second and third pass hit in cache for UNet-sized units).
 template <typename T, bool SILU>
 __global__ __launch_bounds__(kGenericThreads) void gn_generic_kernel(
-    const T *x, T *y, const float *__restrict__ gamma, const float *__restrict__ beta,
-    uint32_t unit_size, uint32_t hw, uint32_t groups, uint32_t ch_per_group, float eps) {
+    const T *x, const T *chunk, T *y, const float *__restrict__ gamma,
+    const float *__restrict__ beta, uint32_t unit_size, uint32_t hw, uint32_t groups,
+    uint32_t ch_per_group, float eps) {
     __shared__ float red_a[kGenericThreads / kWave];
     __shared__ float red_b[kGenericThreads / kWave];
     const uint32_t unit = blockIdx.x;
     const T *xin = x + (size_t)unit * unit_size;
     T *yout = y + (size_t)unit * unit_size;
+    const uint32_t ch0 = (unit % groups) * ch_per_group;
+    const T *cb = chunk ? chunk + (size_t)(unit / groups) * (groups * ch_per_group) + ch0 : nullptr;
+    // element i of the unit, with the optional addend, rounded to the storage type
+    auto value = [&](uint32_t i) {
+        float v = Store<T>::load1(xin + i);
+        if (cb) v = round_to_storage<T>(v + Store<T>::load1(cb + i / hw));
+        return v;
+    };
     float s = 0.0f;
-    for (uint32_t i = threadIdx.x; i < unit_size; i += kGenericThreads) s += Store<T>::load1(xin + i);
+    for (uint32_t i = threadIdx.x; i < unit_size; i += kGenericThreads) s += value(i);
     const float mean = block_sum_rt(s, red_a) / (float)unit_size;
     float q = 0.0f;
     for (uint32_t i = threadIdx.x; i < unit_size; i += kGenericThreads) {
-        const float d = Store<T>::load1(xin + i) - mean;
+        const float d = value(i) - mean;
         q = fmaf(d, d, q);
     }
     const float rstd = 1.0f / sqrtf(block_sum_rt(q, red_b) / (float)unit_size + eps);
-    const uint32_t ch0 = (unit % groups) * ch_per_group;
+    // every lane re-reads only elements it writes itself, so y may alias x
     for (uint32_t i = threadIdx.x; i < unit_size; i += kGenericThreads) {
         const uint32_t c = ch0 + i / hw;
-        const float t = fmaf(Store<T>::load1(xin + i) - mean, rstd * gamma[c], beta[c]);
+        const float t = fmaf(value(i) - mean, rstd * gamma[c], beta[c]);
         Store<T>::store1(yout + i, SILU ? silu_f(t) : t);
     }
 }
@@ -320,22 +345,23 @@ GnPlan plan_slice(uint32_t vecs, uint32_t split, uint32_t force_threads, uint32_
 }
 
 template <typename T, int K>
-void gn_launch_k(bool silu, uint32_t blocks, uint32_t threads, hipStream_t stream, const T *x, T *y,
-                 const float *gamma, const float *beta, const GnScratch &sc, const GnParams &p) {
+void gn_launch_k(bool silu, uint32_t blocks, uint32_t threads, hipStream_t stream, const T *x,
+                 const T *chunk, T *y, const float *gamma, const float *beta, const GnScratch &sc,
+                 const GnParams &p) {
     if (silu)
         hipLaunchKernelGGL((gn_slice_kernel<T, K, true>), dim3(blocks), dim3(threads), 0, stream, x,
-                           y, gamma, beta, sc, p);
+                           chunk, y, gamma, beta, sc, p);
     else
         hipLaunchKernelGGL((gn_slice_kernel<T, K, false>), dim3(blocks), dim3(threads), 0, stream,
-                           x, y, gamma, beta, sc, p);
+                           x, chunk, y, gamma, beta, sc, p);
 }
 
 template <typename T>
-int gn_generic(bool silu, const T *x, T *y, const float *gamma, const float *beta, size_t units,
-               size_t unit_size, size_t hw, size_t groups, size_t cpg, float eps,
+int gn_generic(bool silu, const T *x, const T *chunk, T *y, const float *gamma, const float *beta,
+               size_t units, size_t unit_size, size_t hw, size_t groups, size_t cpg, float eps,
                hipStream_t stream) {
     hipLaunchKernelGGL((silu ? gn_generic_kernel<T, true> : gn_generic_kernel<T, false>),
-                       dim3((uint32_t)units), dim3(kGenericThreads), 0, stream, x, y, gamma, beta,
+                       dim3((uint32_t)units), dim3(kGenericThreads), 0, stream, x, chunk, y, gamma, beta,
                        (uint32_t)unit_size, (uint32_t)hw, (uint32_t)groups, (uint32_t)cpg, eps);
     return launch_status();
 }
@@ -343,11 +369,12 @@ int gn_generic(bool silu, const T *x, T *y, const float *gamma, const float *bet
 }  // namespace
 
 template <typename T>
-int gn_dispatch(const void *xv, void *yv, const float *gamma, const float *beta, size_t batch,
-                size_t channels, size_t hw, size_t groups, float eps, bool silu,
+int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma, const float *beta,
+                size_t batch, size_t channels, size_t hw, size_t groups, float eps, bool silu,
                 hipStream_t stream) {
     constexpr int EPV = Store<T>::EPV;
     const T *x = static_cast<const T *>(xv);
+    const T *chunk = static_cast<const T *>(chunkv);
     T *y = static_cast<T *>(yv);
     const size_t cpg = channels / groups;
     const size_t unit_size = cpg * hw;
@@ -355,7 +382,7 @@ int gn_dispatch(const void *xv, void *yv, const float *gamma, const float *beta,
     if (units == 0 || unit_size == 0) return MSD_OK;
     if (units > 0x7FFFFFFFull || unit_size > 0x7FFFFFFFull) return MSD_ERR_INVALID_VALUE;
     if (!(aligned16(x) && aligned16(y) && hw % EPV == 0))
-        return gn_generic<T>(silu, x, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
+        return gn_generic<T>(silu, x, chunk, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
 
     const size_t vec_per_unit = unit_size / EPV;
     // vectors per lane that stay in registers without spilling under the 1024-lane bound
@@ -366,7 +393,7 @@ int gn_dispatch(const void *xv, void *yv, const float *gamma, const float *beta,
     while ((size_t)split * slice_cap < vec_per_unit && split <= kGnMaxSplit) split *= 2;
     const bool can_split = units <= kGnMaxUnits;
     if (split > kGnMaxSplit || (split > 1 && !can_split))
-        return gn_generic<T>(silu, x, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
+        return gn_generic<T>(silu, x, chunk, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
     if (g_tuning.gn_split > 0) {
         uint32_t forced = (uint32_t)g_tuning.gn_split;
         if (forced > split && can_split && (forced & (forced - 1)) == 0 && forced <= kGnMaxSplit &&
@@ -398,7 +425,7 @@ int gn_dispatch(const void *xv, void *yv, const float *gamma, const float *beta,
     p.inv_count = 1.0f / (float)unit_size;
     // every slice must own at least one vector (ceil division can starve the last ones)
     if ((size_t)p.vec_per_slice * (split - 1) >= vec_per_unit)
-        return gn_generic<T>(silu, x, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
+        return gn_generic<T>(silu, x, chunk, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
 
     uint32_t force_threads = 0;
     if (g_tuning.gn_threads >= kWave && g_tuning.gn_threads <= kGnMaxThreads &&
@@ -407,7 +434,7 @@ int gn_dispatch(const void *xv, void *yv, const float *gamma, const float *beta,
         force_threads = (uint32_t)g_tuning.gn_threads;
     const GnPlan pl = plan_slice(p.vec_per_slice, split, force_threads, kMaxK);
     if (pl.k == 0)
-        return gn_generic<T>(silu, x, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
+        return gn_generic<T>(silu, x, chunk, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
 
     GnScratch sc{nullptr, nullptr, nullptr, nullptr, nullptr};
     if (split > 1) {
@@ -416,23 +443,23 @@ int gn_dispatch(const void *xv, void *yv, const float *gamma, const float *beta,
     }
     const uint32_t blocks = (uint32_t)(units * split);
     switch (pl.k) {
-        case 1: gn_launch_k<T, 1>(silu, blocks, pl.threads, stream, x, y, gamma, beta, sc, p); break;
-        case 2: gn_launch_k<T, 2>(silu, blocks, pl.threads, stream, x, y, gamma, beta, sc, p); break;
-        case 3: gn_launch_k<T, 3>(silu, blocks, pl.threads, stream, x, y, gamma, beta, sc, p); break;
-        case 4: gn_launch_k<T, 4>(silu, blocks, pl.threads, stream, x, y, gamma, beta, sc, p); break;
-        case 5: gn_launch_k<T, 5>(silu, blocks, pl.threads, stream, x, y, gamma, beta, sc, p); break;
-        case 6: gn_launch_k<T, 6>(silu, blocks, pl.threads, stream, x, y, gamma, beta, sc, p); break;
-        case 8: gn_launch_k<T, 8>(silu, blocks, pl.threads, stream, x, y, gamma, beta, sc, p); break;
-        case 10: gn_launch_k<T, 10>(silu, blocks, pl.threads, stream, x, y, gamma, beta, sc, p); break;
-        case 12: gn_launch_k<T, 12>(silu, blocks, pl.threads, stream, x, y, gamma, beta, sc, p); break;
-        default: gn_launch_k<T, 16>(silu, blocks, pl.threads, stream, x, y, gamma, beta, sc, p); break;
+        case 1: gn_launch_k<T, 1>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 2: gn_launch_k<T, 2>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 3: gn_launch_k<T, 3>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 4: gn_launch_k<T, 4>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 5: gn_launch_k<T, 5>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 6: gn_launch_k<T, 6>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 8: gn_launch_k<T, 8>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 10: gn_launch_k<T, 10>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 12: gn_launch_k<T, 12>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        default: gn_launch_k<T, 16>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
     }
     return launch_status();
 }
 
-template int gn_dispatch<float>(const void *, void *, const float *, const float *, size_t, size_t,
-                                size_t, size_t, float, bool, hipStream_t);
-template int gn_dispatch<__half>(const void *, void *, const float *, const float *, size_t, size_t,
-                                 size_t, size_t, float, bool, hipStream_t);
+template int gn_dispatch<float>(const void *, const void *, void *, const float *, const float *,
+                                size_t, size_t, size_t, size_t, float, bool, hipStream_t);
+template int gn_dispatch<__half>(const void *, const void *, void *, const float *, const float *,
+                                 size_t, size_t, size_t, size_t, float, bool, hipStream_t);
 
 }  // namespace msd

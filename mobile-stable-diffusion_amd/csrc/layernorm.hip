@@ -65,8 +65,8 @@ struct Chunk {
 // the gamma / beta of the same columns, all requested before the first use.
 template <typename T, int NW, int VPL, int TL>
 __global__ __launch_bounds__(kLnMaxThreads) void ln_team_kernel(
-    const T *x, T *y, const float *__restrict__ gamma, const float *__restrict__ beta,
-    uint32_t rows, float eps, float inv_dim) {
+    const T *x, const T *res, T *sum, T *y, const float *__restrict__ gamma,
+    const float *__restrict__ beta, uint32_t rows, float eps, float inv_dim) {
     typedef Chunk<T, NW> C;
     typedef typename C::vec_t vec_t;
     constexpr int N = C::N;
@@ -84,6 +84,12 @@ __global__ __launch_bounds__(kLnMaxThreads) void ln_team_kernel(
     vec_t raw[VPL];
 #pragma unroll
     for (int k = 0; k < VPL; k++) raw[k] = __builtin_nontemporal_load(xin + k * TL + j);
+    vec_t raw_res[VPL];
+    if (res != nullptr) {  // uniform: residual to add before the norm (the reference's elemwise_add)
+        const vec_t *rin = reinterpret_cast<const vec_t *>(res) + row_chunk;
+#pragma unroll
+        for (int k = 0; k < VPL; k++) raw_res[k] = __builtin_nontemporal_load(rin + k * TL + j);
+    }
     float g[VPL][N], b[VPL][N];
 #pragma unroll
     for (int k = 0; k < VPL; k++) {
@@ -109,6 +115,21 @@ __global__ __launch_bounds__(kLnMaxThreads) void ln_team_kernel(
         }
     }
     float f[VPL][N];
+    if (res != nullptr) {
+        // x + res, rounded to the storage type and written out exactly as a separate add kernel
+        // would have left it; the norm then works on those stored values
+        vec_t *sout = reinterpret_cast<vec_t *>(sum) + row_chunk;
+#pragma unroll
+        for (int k = 0; k < VPL; k++) {
+            float r[N];
+            C::unpack(raw[k], f[k]);
+            C::unpack(raw_res[k], r);
+#pragma unroll
+            for (int e = 0; e < N; e++) f[k][e] += r[e];
+            raw[k] = C::pack(f[k]);
+            if (live) __builtin_nontemporal_store(raw[k], sout + k * TL + j);
+        }
+    }
     float s = 0.0f;
 #pragma unroll
     for (int k = 0; k < VPL; k++) {
@@ -139,13 +160,20 @@ __global__ __launch_bounds__(kLnMaxThreads) void ln_team_kernel(
 // Any dim: one wavefront per row, scalar accesses, three passes.
 template <typename T>
 __global__ __launch_bounds__(kLnThreads) void ln_generic_kernel(
-    const T *x, T *y, const float *__restrict__ gamma,
+    const T *x, const T *res, T *sum, T *y, const float *__restrict__ gamma,
     const float *__restrict__ beta, uint32_t rows, uint32_t dim, float eps) {
     const uint32_t lane = threadIdx.x & (kWave - 1);
     const uint32_t row = blockIdx.x * (kLnThreads / kWave) + threadIdx.x / kWave;
     if (row >= rows) return;  // whole wavefront leaves together
     const T *xin = x + (size_t)row * dim;
     T *yout = y + (size_t)row * dim;
+    if (res != nullptr) {  // write x + res first; each lane later re-reads only what it wrote
+        const T *rin = res + (size_t)row * dim;
+        T *sout = sum + (size_t)row * dim;
+        for (uint32_t i = lane; i < dim; i += kWave)
+            Store<T>::store1(sout + i, Store<T>::load1(xin + i) + Store<T>::load1(rin + i));
+        xin = sout;
+    }
     float s = 0.0f;
     for (uint32_t i = lane; i < dim; i += kWave) s += Store<T>::load1(xin + i);
     const float mean = wave_sum(s) / (float)dim;
@@ -163,35 +191,35 @@ __global__ __launch_bounds__(kLnThreads) void ln_generic_kernel(
 
 // ---- LayerNorm dispatch ----------------------------------------------------
 template <typename T, int NW, int VPL, int TL>
-void ln_launch(const T *x, T *y, const float *gamma, const float *beta, uint32_t rows, float eps,
-               float inv_dim, hipStream_t stream) {
+void ln_launch(const T *x, const T *res, T *sum, T *y, const float *gamma, const float *beta,
+               uint32_t rows, float eps, float inv_dim, hipStream_t stream) {
     const uint32_t threads = g_tuning.ln_threads ? (uint32_t)g_tuning.ln_threads : (uint32_t)kLnThreads;
     const uint32_t rows_per_block = (kWave / TL) * (threads / kWave);
     const uint32_t blocks = (rows + rows_per_block - 1) / rows_per_block;
-    hipLaunchKernelGGL((ln_team_kernel<T, NW, VPL, TL>), dim3(blocks), dim3(threads), 0, stream, x, y,
-                       gamma, beta, rows, eps, inv_dim);
+    hipLaunchKernelGGL((ln_team_kernel<T, NW, VPL, TL>), dim3(blocks), dim3(threads), 0, stream, x,
+                       res, sum, y, gamma, beta, rows, eps, inv_dim);
 }
 
 template <typename T, int NW, int TL>
-bool ln_launch_vpl(uint32_t vpl, const T *x, T *y, const float *gamma, const float *beta,
-                   uint32_t rows, float eps, float inv_dim, hipStream_t stream) {
+bool ln_launch_vpl(uint32_t vpl, const T *x, const T *res, T *sum, T *y, const float *gamma,
+                   const float *beta, uint32_t rows, float eps, float inv_dim, hipStream_t stream) {
     switch (vpl) {
-        case 1: ln_launch<T, NW, 1, TL>(x, y, gamma, beta, rows, eps, inv_dim, stream); return true;
-        case 2: ln_launch<T, NW, 2, TL>(x, y, gamma, beta, rows, eps, inv_dim, stream); return true;
-        case 3: ln_launch<T, NW, 3, TL>(x, y, gamma, beta, rows, eps, inv_dim, stream); return true;
-        case 4: ln_launch<T, NW, 4, TL>(x, y, gamma, beta, rows, eps, inv_dim, stream); return true;
-        case 5: ln_launch<T, NW, 5, TL>(x, y, gamma, beta, rows, eps, inv_dim, stream); return true;
-        case 6: ln_launch<T, NW, 6, TL>(x, y, gamma, beta, rows, eps, inv_dim, stream); return true;
-        case 7: ln_launch<T, NW, 7, TL>(x, y, gamma, beta, rows, eps, inv_dim, stream); return true;
-        case 8: ln_launch<T, NW, 8, TL>(x, y, gamma, beta, rows, eps, inv_dim, stream); return true;
+        case 1: ln_launch<T, NW, 1, TL>(x, res, sum, y, gamma, beta, rows, eps, inv_dim, stream); return true;
+        case 2: ln_launch<T, NW, 2, TL>(x, res, sum, y, gamma, beta, rows, eps, inv_dim, stream); return true;
+        case 3: ln_launch<T, NW, 3, TL>(x, res, sum, y, gamma, beta, rows, eps, inv_dim, stream); return true;
+        case 4: ln_launch<T, NW, 4, TL>(x, res, sum, y, gamma, beta, rows, eps, inv_dim, stream); return true;
+        case 5: ln_launch<T, NW, 5, TL>(x, res, sum, y, gamma, beta, rows, eps, inv_dim, stream); return true;
+        case 6: ln_launch<T, NW, 6, TL>(x, res, sum, y, gamma, beta, rows, eps, inv_dim, stream); return true;
+        case 7: ln_launch<T, NW, 7, TL>(x, res, sum, y, gamma, beta, rows, eps, inv_dim, stream); return true;
+        case 8: ln_launch<T, NW, 8, TL>(x, res, sum, y, gamma, beta, rows, eps, inv_dim, stream); return true;
         default: return false;
     }
 }
 
 // Tries the team kernel with NW-dword chunks; false when the row does not decompose.
 template <typename T, int NW>
-bool ln_try(const T *x, T *y, const float *gamma, const float *beta, uint32_t rows, uint32_t dim,
-            float eps, float inv_dim, hipStream_t stream) {
+bool ln_try(const T *x, const T *res, T *sum, T *y, const float *gamma, const float *beta,
+            uint32_t rows, uint32_t dim, float eps, float inv_dim, hipStream_t stream) {
     constexpr uint32_t N = NW * 4 / sizeof(T);
     if (dim % N != 0) return false;
     const uint32_t chunks = dim / N;
@@ -199,11 +227,11 @@ bool ln_try(const T *x, T *y, const float *gamma, const float *beta, uint32_t ro
     while (chunks % tl != 0) tl /= 2;
     const uint32_t vpl = chunks / tl;
     switch (tl) {
-        case 64: return ln_launch_vpl<T, NW, 64>(vpl, x, y, gamma, beta, rows, eps, inv_dim, stream);
-        case 32: return ln_launch_vpl<T, NW, 32>(vpl, x, y, gamma, beta, rows, eps, inv_dim, stream);
-        case 16: return ln_launch_vpl<T, NW, 16>(vpl, x, y, gamma, beta, rows, eps, inv_dim, stream);
-        case 8: return ln_launch_vpl<T, NW, 8>(vpl, x, y, gamma, beta, rows, eps, inv_dim, stream);
-        case 4: return ln_launch_vpl<T, NW, 4>(vpl, x, y, gamma, beta, rows, eps, inv_dim, stream);
+        case 64: return ln_launch_vpl<T, NW, 64>(vpl, x, res, sum, y, gamma, beta, rows, eps, inv_dim, stream);
+        case 32: return ln_launch_vpl<T, NW, 32>(vpl, x, res, sum, y, gamma, beta, rows, eps, inv_dim, stream);
+        case 16: return ln_launch_vpl<T, NW, 16>(vpl, x, res, sum, y, gamma, beta, rows, eps, inv_dim, stream);
+        case 8: return ln_launch_vpl<T, NW, 8>(vpl, x, res, sum, y, gamma, beta, rows, eps, inv_dim, stream);
+        case 4: return ln_launch_vpl<T, NW, 4>(vpl, x, res, sum, y, gamma, beta, rows, eps, inv_dim, stream);
         default: return false;
     }
 }
@@ -211,16 +239,19 @@ bool ln_try(const T *x, T *y, const float *gamma, const float *beta, uint32_t ro
 }  // namespace
 
 template <typename T>
-int ln_dispatch(const void *xv, void *yv, const float *gamma, const float *beta, size_t rows,
-                size_t dim, float eps, hipStream_t stream) {
+int ln_dispatch(const void *xv, const void *resv, void *sumv, void *yv, const float *gamma,
+                const float *beta, size_t rows, size_t dim, float eps, hipStream_t stream) {
     const T *x = static_cast<const T *>(xv);
+    const T *res = static_cast<const T *>(resv);
+    T *sum = static_cast<T *>(sumv);
     T *y = static_cast<T *>(yv);
     if (rows == 0 || dim == 0) return MSD_OK;
     if (rows > 0x7FFFFFFFull || dim > 0x7FFFFFFFull) return MSD_ERR_INVALID_VALUE;
     const float inv_dim = 1.0f / (float)dim;
     const uint32_t r = (uint32_t)rows, d = (uint32_t)dim;
     bool done = false;
-    if (aligned16(x) && aligned16(y) && aligned16(gamma) && aligned16(beta)) {
+    if (aligned16(x) && aligned16(y) && aligned16(gamma) && aligned16(beta) &&
+        (res == nullptr || (aligned16(res) && aligned16(sum)))) {
         // A lane's dependent chain (convert, two reductions, affine) is on the critical path
         // of a launch this short, so half-precision rows are spread over more lanes with
         // 8-byte chunks when 16-byte ones would leave a team of fewer than 64 lanes with more
@@ -235,23 +266,23 @@ int ln_dispatch(const void *xv, void *yv, const float *gamma, const float *beta,
         }
         if (g_tuning.ln_chunk == 8) prefer8 = true;
         if (g_tuning.ln_chunk == 16) prefer8 = false;
-        if (prefer8) done = ln_try<T, 2>(x, y, gamma, beta, r, d, eps, inv_dim, stream);
-        if (!done) done = ln_try<T, 4>(x, y, gamma, beta, r, d, eps, inv_dim, stream);
-        if (!done && !prefer8) done = ln_try<T, 2>(x, y, gamma, beta, r, d, eps, inv_dim, stream);
+        if (prefer8) done = ln_try<T, 2>(x, res, sum, y, gamma, beta, r, d, eps, inv_dim, stream);
+        if (!done) done = ln_try<T, 4>(x, res, sum, y, gamma, beta, r, d, eps, inv_dim, stream);
+        if (!done && !prefer8) done = ln_try<T, 2>(x, res, sum, y, gamma, beta, r, d, eps, inv_dim, stream);
     }
     if (!done) {
         const uint32_t rows_per_block = kLnThreads / kWave;
         hipLaunchKernelGGL((ln_generic_kernel<T>),
                            dim3((uint32_t)((rows + rows_per_block - 1) / rows_per_block)),
-                           dim3(kLnThreads), 0, stream, x, y, gamma, beta, (uint32_t)rows,
+                           dim3(kLnThreads), 0, stream, x, res, sum, y, gamma, beta, (uint32_t)rows,
                            (uint32_t)dim, eps);
     }
     return launch_status();
 }
 
-template int ln_dispatch<float>(const void *, void *, const float *, const float *, size_t, size_t,
-                                float, hipStream_t);
-template int ln_dispatch<__half>(const void *, void *, const float *, const float *, size_t, size_t,
-                                 float, hipStream_t);
+template int ln_dispatch<float>(const void *, const void *, void *, void *, const float *,
+                                const float *, size_t, size_t, float, hipStream_t);
+template int ln_dispatch<__half>(const void *, const void *, void *, void *, const float *,
+                                 const float *, size_t, size_t, float, hipStream_t);
 
 }  // namespace msd

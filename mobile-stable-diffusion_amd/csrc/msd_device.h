@@ -63,6 +63,18 @@ struct Store<__half> {
     static __device__ __forceinline__ void store1(__half *p, float v) { *p = __float2half_rn(v); }
 };
 
+// v as the storage type would hold it (identity for float, round-to-nearest-even for half)
+template <typename T>
+__device__ __forceinline__ float round_to_storage(float v);
+template <>
+__device__ __forceinline__ float round_to_storage<float>(float v) {
+    return v;
+}
+template <>
+__device__ __forceinline__ float round_to_storage<__half>(float v) {
+    return __half2float(__float2half_rn(v));
+}
+
 // Streaming (read-once / write-once) 16-byte access.
 __device__ __forceinline__ u32x4 load_stream(const u32x4 *p) {
     return __builtin_nontemporal_load(p);

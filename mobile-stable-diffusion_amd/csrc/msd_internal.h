@@ -40,12 +40,16 @@ extern Tuning g_tuning;
 
 // ---- per-dtype dispatchers (T = float or __half), defined in the kernel files ----
 template <typename T>
-int gn_dispatch(const void *x, void *y, const float *gamma, const float *beta, size_t batch,
-                size_t channels, size_t hw, size_t groups, float eps, bool silu,
+int gn_dispatch(const void *x, const void *chunk, void *y, const float *gamma, const float *beta,
+                size_t batch, size_t channels, size_t hw, size_t groups, float eps, bool silu,
                 hipStream_t stream);
+// res / sum may be null (plain LayerNorm); otherwise sum = x + res is written and normalised
 template <typename T>
-int ln_dispatch(const void *x, void *y, const float *gamma, const float *beta, size_t rows,
-                size_t dim, float eps, hipStream_t stream);
+int ln_dispatch(const void *x, const void *res, void *sum, void *y, const float *gamma,
+                const float *beta, size_t rows, size_t dim, float eps, hipStream_t stream);
+template <typename T>
+int add_dispatch(const void *a, const void *b, void *c, size_t n, size_t chunk_size,
+                 hipStream_t stream);  // chunk_size 0: elementwise; else b holds one value per chunk
 template <typename T>
 int geglu_dispatch(const void *proj, void *out, size_t rows, size_t inner, hipStream_t stream);
 

@@ -23,4 +23,18 @@ int quick_gelu(hipStream_t stream, const DeviceBuffer &src, DeviceBuffer &dst) {
     return run(msd_quick_gelu, stream, src, dst);
 }
 
+int elemwise_add(hipStream_t stream, const DeviceBuffer &a, const DeviceBuffer &b, DeviceBuffer &c) {
+    if (b.bytes() != a.bytes() || c.bytes() != a.bytes() || b.dtype() != a.dtype() || c.dtype() != a.dtype())
+        throw std::runtime_error("operand sizes / types differ");
+    return msd_elemwise_add(a.ptr(), b.ptr(), c.ptr(), a.count(), (int)a.dtype(), stream);
+}
+
+int chunkwise_add(hipStream_t stream, const DeviceBuffer &a, const DeviceBuffer &chunk, DeviceBuffer &c,
+                  size_t chunk_size) {
+    if (c.bytes() != a.bytes() || c.dtype() != a.dtype() || chunk.dtype() != a.dtype() || chunk_size == 0 ||
+        a.count() % chunk_size != 0 || chunk.count() != a.count() / chunk_size)
+        throw std::runtime_error("chunk size does not match the operand");
+    return msd_chunkwise_add(a.ptr(), chunk.ptr(), c.ptr(), a.count(), chunk_size, (int)a.dtype(), stream);
+}
+
 }  // namespace msd

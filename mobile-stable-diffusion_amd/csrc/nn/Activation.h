@@ -16,4 +16,10 @@ int silu(hipStream_t stream, const DeviceBuffer &src, DeviceBuffer &dst);       
 int gelu(hipStream_t stream, const DeviceBuffer &src, DeviceBuffer &dst);        // K/util.cl:104-122
 int quick_gelu(hipStream_t stream, const DeviceBuffer &src, DeviceBuffer &dst);  // x*sigmoid(1.702x)
 
+// The two additions of the reference's utility kernels, for call sites that are not fused into
+// a norm: c = a + b (K/util.cl:1-12) and c[i] = a[i] + chunk[i / chunk_size] (K/util.cl:136-148).
+int elemwise_add(hipStream_t stream, const DeviceBuffer &a, const DeviceBuffer &b, DeviceBuffer &c);
+int chunkwise_add(hipStream_t stream, const DeviceBuffer &a, const DeviceBuffer &chunk, DeviceBuffer &c,
+                  size_t chunk_size);
+
 }  // namespace msd

@@ -49,6 +49,19 @@ void GroupNorm::checkInput(size_t input_bytes, DType dtype) const {
 
 int GroupNorm::forward(const DeviceBuffer &input, DeviceBuffer &output, unsigned num_events_in_list,
                        const hipEvent_t *event_wait_list, hipEvent_t event) {
+    return run(input, nullptr, output, num_events_in_list, event_wait_list, event);
+}
+
+int GroupNorm::forward(const DeviceBuffer &input, const DeviceBuffer &chunk, DeviceBuffer &output,
+                       unsigned num_events_in_list, const hipEvent_t *event_wait_list,
+                       hipEvent_t event) {
+    if (chunk.dtype() != input.dtype() || chunk.count() != batch * num_channels)
+        throw std::runtime_error("chunk size != batch * num_channels");
+    return run(input, &chunk, output, num_events_in_list, event_wait_list, event);
+}
+
+int GroupNorm::run(const DeviceBuffer &input, const DeviceBuffer *chunk, DeviceBuffer &output,
+                   unsigned num_events_in_list, const hipEvent_t *event_wait_list, hipEvent_t event) {
     if (bufferWeight.empty() || bufferBias.empty()) throw std::runtime_error("GroupNorm: init() not called");
     checkInput(input.bytes(), input.dtype());
     if (output.bytes() != input.bytes() || output.dtype() != input.dtype())
@@ -59,10 +72,14 @@ int GroupNorm::forward(const DeviceBuffer &input, DeviceBuffer &output, unsigned
     }
     const size_t input_size = input.count() / batch;
     const size_t channelSize = input_size / num_channels;  // H*W (M/nn/GroupNorm.cpp:130)
-    const int rc = msd_groupnorm(input.ptr(), output.ptr(), static_cast<const float *>(bufferWeight.ptr()),
-                                 static_cast<const float *>(bufferBias.ptr()), batch, num_channels,
-                                 channelSize, num_groups, eps, fuse_silu ? 1 : 0, (int)input.dtype(),
-                                 stream);
+    const float *w = static_cast<const float *>(bufferWeight.ptr());
+    const float *b = static_cast<const float *>(bufferBias.ptr());
+    const int rc = chunk ? msd_chunk_add_groupnorm(input.ptr(), chunk->ptr(), output.ptr(), w, b, batch,
+                                                   num_channels, channelSize, num_groups, eps,
+                                                   fuse_silu ? 1 : 0, (int)input.dtype(), stream)
+                         : msd_groupnorm(input.ptr(), output.ptr(), w, b, batch, num_channels,
+                                         channelSize, num_groups, eps, fuse_silu ? 1 : 0,
+                                         (int)input.dtype(), stream);
     if (rc != MSD_OK) return rc;
     if (event) return (int)hipEventRecord(event, stream);
     return MSD_OK;

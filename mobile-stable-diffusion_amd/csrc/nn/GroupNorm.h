@@ -41,10 +41,21 @@ public:
     int forward(const DeviceBuffer &input, DeviceBuffer &output, unsigned num_events_in_list = 0,
                 const hipEvent_t *event_wait_list = nullptr, hipEvent_t event = nullptr);
 
+    // forward() on input + chunk, chunk = one value per (sample, channel) broadcast over H*W:
+    // the chunkwise_add the reference's ResBlock runs right before its out-norm
+    // (M/nn/ResBlock.cpp:188-199, then :222) folded into the same launch.  The result equals
+    // chunkwise_add followed by forward() bit for bit.  chunk holds batch * num_channels
+    // elements of the input's storage type.
+    int forward(const DeviceBuffer &input, const DeviceBuffer &chunk, DeviceBuffer &output,
+                unsigned num_events_in_list = 0, const hipEvent_t *event_wait_list = nullptr,
+                hipEvent_t event = nullptr);
+
     // The precondition checks of forward() alone (no device work).
     void checkInput(size_t input_bytes, DType dtype) const;
 
 private:
+    int run(const DeviceBuffer &input, const DeviceBuffer *chunk, DeviceBuffer &output,
+            unsigned num_events_in_list, const hipEvent_t *event_wait_list, hipEvent_t event);
     DeviceBuffer bufferWeight;
     DeviceBuffer bufferBias;
     size_t weightSize;

@@ -57,4 +57,25 @@ int LayerNorm::forward(const DeviceBuffer &input, DeviceBuffer &output, unsigned
     return MSD_OK;
 }
 
+int LayerNorm::forwardAdd(const DeviceBuffer &a, const DeviceBuffer &b, DeviceBuffer &sum,
+                          DeviceBuffer &output, unsigned num_events_in_list,
+                          const hipEvent_t *event_wait_list, hipEvent_t event) {
+    if (bufferWeight.empty() || bufferBias.empty()) throw std::runtime_error("LayerNorm: init() not called");
+    checkInput(a.bytes(), a.dtype());
+    if (b.bytes() != a.bytes() || sum.bytes() != a.bytes() || output.bytes() != a.bytes() ||
+        b.dtype() != a.dtype() || sum.dtype() != a.dtype() || output.dtype() != a.dtype())
+        throw std::runtime_error("operand sizes / types differ");
+    for (unsigned i = 0; i < num_events_in_list; i++) {
+        const hipError_t err = hipStreamWaitEvent(stream, event_wait_list[i], 0);
+        if (err != hipSuccess) return (int)err;
+    }
+    const int rc = msd_add_layernorm(a.ptr(), b.ptr(), sum.ptr(), output.ptr(),
+                                     static_cast<const float *>(bufferWeight.ptr()),
+                                     static_cast<const float *>(bufferBias.ptr()), a.count() / weightSize,
+                                     weightSize, eps, (int)a.dtype(), stream);
+    if (rc != MSD_OK) return rc;
+    if (event) return (int)hipEventRecord(event, stream);
+    return MSD_OK;
+}
+
 }  // namespace msd

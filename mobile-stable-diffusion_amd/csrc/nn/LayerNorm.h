@@ -29,6 +29,13 @@ public:
     // std::runtime_error("input_size % weight->num_vals != 0").  Returns 0 or a hipError_t.
     int forward(const DeviceBuffer &input, DeviceBuffer &output, unsigned num_events_in_list = 0,
                 const hipEvent_t *event_wait_list = nullptr, hipEvent_t event = nullptr);
+    // sum = a + b, output = LayerNorm(sum) in one launch: the elemwise_add the reference runs
+    // before LayerNorm 2 and 3 (M/nn/BasicTransformerBlock.cpp:126-136,149-158) folded in; `sum`
+    // is written because the block keeps it as its next residual, and may be `a` itself.
+    // Equals elemwise_add followed by forward() bit for bit.
+    int forwardAdd(const DeviceBuffer &a, const DeviceBuffer &b, DeviceBuffer &sum, DeviceBuffer &output,
+                   unsigned num_events_in_list = 0, const hipEvent_t *event_wait_list = nullptr,
+                   hipEvent_t event = nullptr);
     void checkInput(size_t input_bytes, DType dtype) const;
 
 private:

@@ -92,6 +92,13 @@ int msdnn_groupnorm_forward(void *h, void *in, void *out, size_t bytes, int dtyp
         return static_cast<GroupNorm *>(h)->forward(i, o);
     });
 }
+int msdnn_groupnorm_forward_chunk(void *h, void *in, void *chunk, size_t chunk_bytes, void *out, size_t bytes,
+                                  int dtype) {
+    return guarded([&] {
+        DeviceBuffer i = wrap(in, bytes, dtype), c = wrap(chunk, chunk_bytes, dtype), o = wrap(out, bytes, dtype);
+        return static_cast<GroupNorm *>(h)->forward(i, c, o);
+    });
+}
 void msdnn_groupnorm_destroy(void *h) { delete static_cast<GroupNorm *>(h); }
 
 // ---- LayerNorm
@@ -120,6 +127,13 @@ int msdnn_layernorm_forward(void *h, void *in, void *out, size_t bytes, int dtyp
     return guarded([&] {
         DeviceBuffer i = wrap(in, bytes, dtype), o = wrap(out, bytes, dtype);
         return static_cast<LayerNorm *>(h)->forward(i, o);
+    });
+}
+int msdnn_layernorm_forward_add(void *h, void *a, void *b, void *sum, void *out, size_t bytes, int dtype) {
+    return guarded([&] {
+        DeviceBuffer ab = wrap(a, bytes, dtype), bb = wrap(b, bytes, dtype), sb = wrap(sum, bytes, dtype),
+                     ob = wrap(out, bytes, dtype);
+        return static_cast<LayerNorm *>(h)->forwardAdd(ab, bb, sb, ob);
     });
 }
 void msdnn_layernorm_destroy(void *h) { delete static_cast<LayerNorm *>(h); }

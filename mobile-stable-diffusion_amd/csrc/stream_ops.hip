@@ -117,6 +117,38 @@ __global__ __launch_bounds__(kStreamThreads) void act_generic_kernel(const T *x,
         Store<T>::store1(y + i, OP::apply(Store<T>::load1(x + i)));
 }
 
+// c[i] = a[i] + b[i]  (chunk_vecs == 0), or c[i] = a[i] + b[i / chunk] with one b value per
+// chunk of `chunk_vecs` vectors (the per-channel broadcast add).  c may alias a or b.
+template <typename T>
+__global__ __launch_bounds__(kStreamThreads) void add_kernel(const T *a, const T *b, T *c,
+                                                             uint32_t vecs, FastDiv chunk_vecs) {
+    constexpr int EPV = Store<T>::EPV;
+    const uint32_t v = blockIdx.x * kStreamThreads + threadIdx.x;
+    if (v >= vecs) return;
+    float fa[EPV], fb[EPV];
+    Store<T>::unpack(load_stream(reinterpret_cast<const u32x4 *>(a) + v), fa);
+    if (chunk_vecs.d == 0) {
+        Store<T>::unpack(load_stream(reinterpret_cast<const u32x4 *>(b) + v), fb);
+#pragma unroll
+        for (int e = 0; e < EPV; e++) fa[e] += fb[e];
+    } else {
+        const float bv = Store<T>::load1(b + fast_div(v, chunk_vecs));
+#pragma unroll
+        for (int e = 0; e < EPV; e++) fa[e] += bv;
+    }
+    store_stream(reinterpret_cast<u32x4 *>(c) + v, Store<T>::pack(fa));
+}
+
+template <typename T>
+__global__ __launch_bounds__(kStreamThreads) void add_generic_kernel(const T *a, const T *b, T *c,
+                                                                     size_t n, size_t chunk_size) {
+    for (size_t i = (size_t)blockIdx.x * kStreamThreads + threadIdx.x; i < n;
+         i += (size_t)gridDim.x * kStreamThreads) {
+        const float bv = Store<T>::load1(b + (chunk_size ? i / chunk_size : i));
+        Store<T>::store1(c + i, Store<T>::load1(a + i) + bv);
+    }
+}
+
 // ---------------------------------------------------------------------------
 // Timestep embedding
 // ---------------------------------------------------------------------------
@@ -214,6 +246,30 @@ int act_launch(const void *xv, void *yv, size_t n, hipStream_t stream) {
 }  // namespace
 
 template <typename T>
+int add_dispatch(const void *av, const void *bv, void *cv, size_t n, size_t chunk_size,
+                 hipStream_t stream) {
+    constexpr int EPV = Store<T>::EPV;
+    const T *a = static_cast<const T *>(av);
+    const T *b = static_cast<const T *>(bv);
+    T *c = static_cast<T *>(cv);
+    if (n == 0) return MSD_OK;
+    const bool vec_ok = aligned16(a) && aligned16(c) && n % EPV == 0 && n / EPV < 0x7FFFFFFFull &&
+                        (chunk_size == 0 ? aligned16(b) : chunk_size % EPV == 0);
+    if (vec_ok) {
+        const uint32_t vecs = (uint32_t)(n / EPV);
+        FastDiv fd = make_fast_div((uint32_t)(chunk_size / EPV));
+        if (chunk_size == 0) fd.d = 0;
+        hipLaunchKernelGGL((add_kernel<T>), dim3((vecs + kStreamThreads - 1) / kStreamThreads),
+                           dim3(kStreamThreads), 0, stream, a, b, c, vecs, fd);
+    } else {
+        const size_t want = (n + kStreamThreads - 1) / kStreamThreads;
+        hipLaunchKernelGGL((add_generic_kernel<T>), dim3((uint32_t)(want < 65536 ? want : 65536)),
+                           dim3(kStreamThreads), 0, stream, a, b, c, n, chunk_size);
+    }
+    return launch_status();
+}
+
+template <typename T>
 int act_dispatch(Act op, const void *x, void *y, size_t n, hipStream_t stream) {
     switch (op) {
         case Act::Silu: return act_launch<T, OpSilu>(x, y, n, stream);
@@ -236,6 +292,8 @@ int temb_dispatch(const int64_t *timesteps, void *out, size_t batch, size_t dim,
 
 template int geglu_dispatch<float>(const void *, void *, size_t, size_t, hipStream_t);
 template int geglu_dispatch<__half>(const void *, void *, size_t, size_t, hipStream_t);
+template int add_dispatch<float>(const void *, const void *, void *, size_t, size_t, hipStream_t);
+template int add_dispatch<__half>(const void *, const void *, void *, size_t, size_t, hipStream_t);
 template int act_dispatch<float>(Act, const void *, void *, size_t, hipStream_t);
 template int act_dispatch<__half>(Act, const void *, void *, size_t, hipStream_t);
 template int temb_dispatch<float>(const int64_t *, void *, size_t, size_t, float, hipStream_t);

@@ -254,6 +254,16 @@ void orc_gelu_multiply(const float *ab, float *dst, size_t rows, size_t inner) {
     }
 }
 
+void orc_elemwise_add(const float *a, const float *b, float *c, size_t n) {
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < n; i++) c[i] = a[i] + b[i]; /* K/util.cl:11 */
+}
+
+void orc_chunkwise_add(const float *a, const float *chunk, float *c, size_t n, size_t chunk_size) {
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < n; i++) c[i] = a[i] + chunk[i / chunk_size]; /* K/util.cl:143-147 */
+}
+
 void orc_timestep_freqs(float *freq, int half, float max_period) {
     for (int i = 0; i < half; i++) /* M/UNetModel.cpp:1950, float overloads throughout */
         freq[i] = expf((-logf(max_period)) * (float)i / (float)half);

@@ -54,6 +54,8 @@ def lib():
         "orc_gelu": (None, [_f32p, _f32p, _sz]),
         "orc_quick_gelu": (None, [_f32p, _f32p, _sz]),
         "orc_gelu_multiply": (None, [_f32p, _f32p, _sz, _sz]),
+        "orc_elemwise_add": (None, [_f32p, _f32p, _f32p, _sz]),
+        "orc_chunkwise_add": (None, [_f32p, _f32p, _f32p, _sz, _sz]),
         "orc_timestep_embedding": (None, [_i64, _f32p, _it, _fl]),
         "orc_timestep_freqs": (None, [_f32p, _it, _fl]),
         "orc_ddim_timesteps": (_it, [_it, _i32p, _it]),
@@ -171,6 +173,22 @@ def geglu(ab):
     y = np.empty(ab.shape[:-1] + (inner,), dtype=np.float32)
     lib().orc_gelu_multiply(ab.reshape(-1), y.reshape(-1), rows, inner)
     return y
+
+
+def elemwise_add(a, b):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    b = np.ascontiguousarray(b, dtype=np.float32)
+    c = np.empty_like(a)
+    lib().orc_elemwise_add(a.reshape(-1), b.reshape(-1), c.reshape(-1), a.size)
+    return c
+
+
+def chunkwise_add(a, chunk, chunk_size):
+    """a: any shape; chunk: flat, one value per run of chunk_size elements of a."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    c = np.empty_like(a)
+    lib().orc_chunkwise_add(a.reshape(-1), _c(chunk), c.reshape(-1), a.size, chunk_size)
+    return c
 
 
 def timestep_embedding(t, dim=320, max_period=10000.0):

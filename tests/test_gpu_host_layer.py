@@ -122,6 +122,46 @@ def test_activations_and_timestep_embedding_through_objects(msd, nn, orc, cuda):
     torch.cuda.synchronize()
 
 
+def test_objects_with_fused_adds(msd, nn, orc, cuda, tmp_path):
+    """ResBlock out-norm with the embedding add, and LayerNorm 2 with the residual add, through
+    the layer objects (M/nn/ResBlock.cpp:188-232, M/nn/BasicTransformerBlock.cpp:126-136)."""
+    import torch
+    channels, hw, batch = 640, 1024, 2
+    w = orc.normal((channels,), seed=41, mean=1.0, sigma=0.1)
+    b = orc.normal((channels,), seed=42, sigma=0.1)
+    np.save(tmp_path / "out_w.npy", w)
+    np.save(tmp_path / "out_b.npy", b)
+    x = orc.round_to_half(orc.normal((batch, channels, hw), seed=43, sigma=1.5))
+    emb = orc.round_to_half(orc.normal((batch, channels), seed=44))
+    g = nn.msdnn_groupnorm_create(None, 32, channels, 1e-5, b"out_w.npy", b"out_b.npy", batch, 1)
+    assert nn.msdnn_groupnorm_init(g) == 0, msd.nn_last_error()
+    xd, ed = _dev(x, cuda, True), _dev(emb, cuda, True)
+    nbytes = xd.numel() * 2
+    assert nn.msdnn_groupnorm_forward_chunk(g, _ptr(xd), _ptr(ed), ed.numel() * 2, _ptr(xd), nbytes, 1) == 0
+    ref = orc.groupnorm(orc.round_to_half(orc.chunkwise_add(x, emb, hw)), w, b, 32, 1e-5, silu=True)
+    assert_close_f16(xd.float().cpu().numpy(), orc.round_to_half(ref))
+    assert nn.msdnn_groupnorm_forward_chunk(g, _ptr(xd), _ptr(ed), ed.numel() * 2 - 2, _ptr(xd), nbytes, 1) < 0
+    assert "chunk size" in msd.nn_last_error()
+    nn.msdnn_groupnorm_destroy(g)
+
+    dim, rows = 640, 2048
+    lw = orc.normal((dim,), seed=45, mean=1.0, sigma=0.1)
+    lb = orc.normal((dim,), seed=46, sigma=0.1)
+    np.save(tmp_path / "n2_w.npy", lw)
+    np.save(tmp_path / "n2_b.npy", lb)
+    a = orc.normal((rows, dim), seed=47)
+    r = orc.normal((rows, dim), seed=48, sigma=2.0)
+    ln = nn.msdnn_layernorm_create(None, dim, b"n2_w.npy", b"n2_b.npy", 1e-5)
+    assert nn.msdnn_layernorm_init(ln) == 0, msd.nn_last_error()
+    ad, rd = _dev(a, cuda), _dev(r, cuda)
+    yd = torch.empty_like(ad)
+    assert nn.msdnn_layernorm_forward_add(ln, _ptr(ad), _ptr(rd), _ptr(ad), _ptr(yd), a.nbytes, 0) == 0
+    s = orc.elemwise_add(a, r)
+    assert np.array_equal(ad.cpu().numpy(), s)  # the sum replaced the first operand
+    assert_close_f32(yd.cpu().numpy(), orc.layernorm(s, lw, lb, 1e-5))
+    nn.msdnn_layernorm_destroy(ln)
+
+
 def test_step_runner_eager_and_graph(msd, nn, cuda):
     import torch
     stream = torch.cuda.Stream()  # graph capture needs a stream of its own, not the default one

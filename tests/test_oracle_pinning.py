@@ -161,6 +161,14 @@ def test_geglu_half_order_and_fixture(orc, golden):
     assert_close_f32(got, orc.geglu64(ab), 2e-6)
 
 
+def test_add_kernels_are_exact(orc):
+    a = orc.normal((2, 6, 5, 7), seed=81, sigma=3.0)
+    b = orc.normal((2, 6, 5, 7), seed=82)
+    assert np.array_equal(orc.elemwise_add(a, b), a + b)
+    chunk = orc.normal((2, 6), seed=83)  # one value per (sample, channel), broadcast over H*W
+    assert np.array_equal(orc.chunkwise_add(a, chunk, 35), a + chunk[:, :, None, None])
+
+
 # ----------------------------------------------------------------- timestep embedding
 def test_timestep_embedding_closed_forms(orc, golden):
     e0 = orc.timestep_embedding(0)
