@@ -247,16 +247,30 @@ def shape_table(torch, msd, dev, stream):
                     else:
                         rc = lib.msd_geglu(vp(x.data_ptr()), vp(y.data_ptr()), p["rows"], p["inner"], code, sp)
                     assert rc == 0
-            replay = capture(torch, msd, stream, body)
-            with torch.cuda.stream(stream):
-                replay()
-                reps = max(2, int(2000 // copies))
-                ms = event_time_ms(torch, replay, reps)
-            us = ms * 1e3 / (reps * copies)
-            gbs = nbytes / us / 1e3
-            rows.append({"kernel": kind, "shape": p, "dtype": "f16" if elt == 2 else "f32",
-                         "bytes": nbytes, "us": round(us, 3), "GBps": round(gbs, 1),
-                         "pct_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 1)})
+            # the same bytes through a plain copy kernel: what a launch of this size can reach
+            in_bytes, out_bytes = n_in * elt, n_out * elt
+
+            def copy_body():
+                sp = vp(torch.cuda.current_stream().cuda_stream)
+                for x, y in zip(xs, ys):
+                    assert lib.msd_copy(vp(x.data_ptr()), vp(y.data_ptr()), out_bytes, sp) == 0
+            reps = max(2, int(2000 // copies))
+            us = {}
+            for name, fn in (("kernel", body), ("copy", copy_body)):
+                if name == "copy" and in_bytes != out_bytes:
+                    continue
+                replay = capture(torch, msd, stream, fn)
+                with torch.cuda.stream(stream):
+                    replay()
+                    us[name] = event_time_ms(torch, replay, reps) * 1e3 / (reps * copies)
+            gbs = nbytes / us["kernel"] / 1e3
+            row = {"kernel": kind, "shape": p, "dtype": "f16" if elt == 2 else "f32",
+                   "bytes": nbytes, "us": round(us["kernel"], 3), "GBps": round(gbs, 1),
+                   "pct_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 1)}
+            if in_bytes == out_bytes:  # one copy launch moves exactly the kernel's bytes
+                row["copy_us"] = round(us["copy"], 3)
+                row["pct_of_copy_rate"] = round(100.0 * us["copy"] / us["kernel"], 1)
+            rows.append(row)
             del xs, ys
             torch.cuda.empty_cache()
     return rows

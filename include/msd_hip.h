@@ -138,6 +138,14 @@ int msd_gelu(const void *x, void *y, size_t n, int dtype, void *stream);
 int msd_quick_gelu(const void *x, void *y, size_t n, int dtype, void *stream);
 
 /*
+ * Plain device copy of `bytes` (multiple of 4) with the same 16-byte streaming kernel the
+ * activations use and no arithmetic.  Measurement helper with no reference counterpart: it
+ * gives the bandwidth a read-once / write-once launch of a given size can reach on the
+ * machine, the ceiling the other kernels are compared with, and calibrates traffic counters.
+ */
+int msd_copy(const void *src, void *dst, size_t bytes, void *stream);
+
+/*
  * Sinusoidal timestep embedding, out[b] = [cos(t_b*f_i) | sin(t_b*f_i)],
  * f_i = exp(-log(max_period) * i / (dim/2)), i < dim/2.  Replaces the host loop
  * UNetModel::createTimestepEmbedding (M/UNetModel.cpp:1935-1958): same float32

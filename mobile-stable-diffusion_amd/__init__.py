@@ -24,7 +24,7 @@ C_ABI_SYMBOLS = (
     "msd_version", "msd_error_string", "msd_init", "msd_shutdown", "msd_status",
     "msd_set_tuning", "msd_groupnorm", "msd_layernorm", "msd_geglu",
     "msd_silu", "msd_gelu", "msd_quick_gelu", "msd_timestep_embedding", "msd_ddim_timesteps",
-    "msd_elemwise_add", "msd_chunkwise_add", "msd_chunk_add_groupnorm", "msd_add_layernorm",
+    "msd_elemwise_add", "msd_chunkwise_add", "msd_chunk_add_groupnorm", "msd_add_layernorm", "msd_copy",
 )
 
 _lib = None
@@ -56,6 +56,7 @@ def load_library(path=None):
     lib.msd_groupnorm.argtypes = [vp, vp, vp, vp, sz, sz, sz, sz, fl, it, it, vp]
     lib.msd_layernorm.argtypes = [vp, vp, vp, vp, sz, sz, fl, it, vp]
     lib.msd_geglu.argtypes = [vp, vp, sz, sz, it, vp]
+    lib.msd_copy.argtypes = [vp, vp, sz, vp]
     lib.msd_elemwise_add.argtypes = [vp, vp, vp, sz, it, vp]
     lib.msd_chunkwise_add.argtypes = [vp, vp, vp, sz, sz, it, vp]
     lib.msd_chunk_add_groupnorm.argtypes = [vp, vp, vp, vp, vp, sz, sz, sz, sz, fl, it, it, vp]

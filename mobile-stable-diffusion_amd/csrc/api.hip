@@ -247,6 +247,11 @@ int msd_quick_gelu(const void *x, void *y, size_t n, int dtype, void *stream) {
     return act_entry(Act::QuickGelu, x, y, n, dtype, stream);
 }
 
+int msd_copy(const void *src, void *dst, size_t bytes, void *stream) {
+    if (bytes % 4 != 0) return MSD_ERR_INVALID_VALUE;
+    return act_entry(Act::Copy, src, dst, bytes / 4, MSD_DTYPE_F32, stream);
+}
+
 int msd_timestep_embedding(const int64_t *timesteps, void *out, size_t batch, size_t dim,
                            float max_period, int dtype, void *stream) {
     if (dim % 2 != 0 || !(max_period > 0.0f)) return MSD_ERR_INVALID_VALUE;

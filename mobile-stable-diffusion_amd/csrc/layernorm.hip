@@ -10,8 +10,7 @@
 namespace msd {
 namespace {
 
-constexpr int kLnThreads = 64;      // default workgroup: one wavefront (measured: never slower
-                                    // than 128 / 256 / 512 lanes, 5 - 8 % faster below 1000 rows)
+constexpr int kLnThreads = 64;      // workgroup of the scalar kernel; smallest team-kernel workgroup
 constexpr int kLnMaxThreads = 512;  // launch bound
 
 // NW dwords (8 or 16 bytes) of T, moved with one instruction.
@@ -193,7 +192,11 @@ __global__ __launch_bounds__(kLnThreads) void ln_generic_kernel(
 template <typename T, int NW, int VPL, int TL>
 void ln_launch(const T *x, const T *res, T *sum, T *y, const float *gamma, const float *beta,
                uint32_t rows, float eps, float inv_dim, hipStream_t stream) {
-    const uint32_t threads = g_tuning.ln_threads ? (uint32_t)g_tuning.ln_threads : (uint32_t)kLnThreads;
+    // one wavefront per workgroup is 2 - 8 % faster while the launch is small (measured below
+    // about 1000 wavefronts); large launches dispatch sooner as 4-wavefront workgroups
+    const uint32_t wavefronts = (rows + (kWave / TL) - 1) / (kWave / TL);
+    const uint32_t threads = g_tuning.ln_threads ? (uint32_t)g_tuning.ln_threads
+                                                 : (wavefronts >= 1024 ? 256u : (uint32_t)kLnThreads);
     const uint32_t rows_per_block = (kWave / TL) * (threads / kWave);
     const uint32_t blocks = (rows + rows_per_block - 1) / rows_per_block;
     hipLaunchKernelGGL((ln_team_kernel<T, NW, VPL, TL>), dim3(blocks), dim3(threads), 0, stream, x,

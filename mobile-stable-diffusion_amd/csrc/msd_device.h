@@ -199,6 +199,9 @@ __device__ __forceinline__ float gelu_erf_f(float x) {
     return x * (x < 0.0f ? half_e : 1.0f - half_e);
 }
 
+struct OpCopy {
+    static __device__ __forceinline__ float apply(float x) { return x; }
+};
 struct OpSilu {
     static __device__ __forceinline__ float apply(float x) { return silu_f(x); }
 };

@@ -53,7 +53,7 @@ int add_dispatch(const void *a, const void *b, void *c, size_t n, size_t chunk_s
 template <typename T>
 int geglu_dispatch(const void *proj, void *out, size_t rows, size_t inner, hipStream_t stream);
 
-enum class Act { Silu, Gelu, QuickGelu };
+enum class Act { Silu, Gelu, QuickGelu, Copy };
 template <typename T>
 int act_dispatch(Act op, const void *x, void *y, size_t n, hipStream_t stream);
 template <typename T>

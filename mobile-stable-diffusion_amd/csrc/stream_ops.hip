@@ -275,6 +275,7 @@ int act_dispatch(Act op, const void *x, void *y, size_t n, hipStream_t stream) {
         case Act::Silu: return act_launch<T, OpSilu>(x, y, n, stream);
         case Act::Gelu: return act_launch<T, OpGelu>(x, y, n, stream);
         case Act::QuickGelu: return act_launch<T, OpQuickGelu>(x, y, n, stream);
+        case Act::Copy: return act_launch<T, OpCopy>(x, y, n, stream);
     }
     return MSD_ERR_INVALID_VALUE;
 }
