@@ -276,6 +276,98 @@ def shape_table(torch, msd, dev, stream):
     return rows
 
 
+def fusion_table(torch, msd, dev, stream):
+    """The additions / permute the reference runs next to its norms, as separate launches and
+    folded into the norm kernel (fp16, batch 2, graph-replayed on rotating cold buffers)."""
+    import ctypes
+    vp = ctypes.c_void_p
+    lib = msd.load_library()
+    F16 = msd.DTYPE_F16
+    rows = []
+
+    def measure(bodies, copies):
+        out = {}
+        for name, fn in bodies.items():
+            replay = capture(torch, msd, stream, fn)
+            with torch.cuda.stream(stream):
+                replay()
+                reps = max(2, int(1500 // copies))
+                out[name] = event_time_ms(torch, replay, reps) * 1e3 / (reps * copies)
+        return out
+
+    def sp():
+        return vp(torch.cuda.current_stream().cuda_stream)
+
+    for c, side in [(320, 64), (640, 32), (1280, 16), (1280, 8)]:
+        hw = side * side
+        n = BATCH * c * hw
+        copies = max(4, min(128, int(400e6 // (4 * n)) + 1))
+        xs = [torch.randn(n, device=dev).half() for _ in range(copies)]
+        ys = [torch.empty(n, device=dev, dtype=torch.float16) for _ in range(copies)]
+        emb = torch.randn(BATCH * c, device=dev).half()
+        ga, be = torch.ones(c, device=dev), torch.zeros(c, device=dev)
+        g, b, e = vp(ga.data_ptr()), vp(be.data_ptr()), vp(emb.data_ptr())
+
+        def add_then_norm():
+            for x in xs:
+                xp = vp(x.data_ptr())
+                assert lib.msd_chunkwise_add(xp, e, xp, n, hw, F16, sp()) == 0
+                assert lib.msd_groupnorm(xp, xp, g, b, BATCH, c, hw, 32, 1e-5, 1, F16, sp()) == 0
+
+        def add_norm_fused():
+            for x in xs:
+                xp = vp(x.data_ptr())
+                assert lib.msd_chunk_add_groupnorm(xp, e, xp, g, b, BATCH, c, hw, 32, 1e-5, 1, F16, sp()) == 0
+
+        def norm_then_permute():
+            for x, y in zip(xs, ys):
+                xp, yp = vp(x.data_ptr()), vp(y.data_ptr())
+                assert lib.msd_groupnorm(xp, xp, g, b, BATCH, c, hw, 32, 1e-6, 0, F16, sp()) == 0
+                assert lib.msd_permute_0_2_1(xp, yp, BATCH, c, hw, F16, sp()) == 0
+
+        def norm_tokens_fused():
+            for x, y in zip(xs, ys):
+                assert lib.msd_groupnorm_tokens(vp(x.data_ptr()), vp(y.data_ptr()), g, b, BATCH, c, hw, 32,
+                                                1e-6, F16, sp()) == 0
+
+        t = measure({"a2": add_then_norm, "a1": add_norm_fused, "p2": norm_then_permute,
+                     "p1": norm_tokens_fused}, copies)
+        rows.append({"what": "chunkwise_add + GroupNorm+SiLU (ResBlock out-norm)", "shape": {"c": c, "hw": hw},
+                     "us_separate": round(t["a2"], 2), "us_fused": round(t["a1"], 2),
+                     "speedup": round(t["a2"] / t["a1"], 2)})
+        rows.append({"what": "GroupNorm + permute to tokens (SpatialTransformer)", "shape": {"c": c, "hw": hw},
+                     "us_separate": round(t["p2"], 2), "us_fused": round(t["p1"], 2),
+                     "speedup": round(t["p2"] / t["p1"], 2)})
+        del xs, ys
+    for r, d in [(8192, 320), (2048, 640), (512, 1280)]:
+        n = r * d
+        copies = max(4, min(128, int(400e6 // (8 * n)) + 1))
+        xs = [torch.randn(n, device=dev).half() for _ in range(copies)]
+        rs = [torch.randn(n, device=dev).half() for _ in range(copies)]
+        ys = [torch.empty(n, device=dev, dtype=torch.float16) for _ in range(copies)]
+        ga, be = torch.ones(d, device=dev), torch.zeros(d, device=dev)
+        g, b = vp(ga.data_ptr()), vp(be.data_ptr())
+
+        def add_then_ln():
+            for x, res, y in zip(xs, rs, ys):
+                xp, rp, yp = vp(x.data_ptr()), vp(res.data_ptr()), vp(y.data_ptr())
+                assert lib.msd_elemwise_add(xp, rp, xp, n, F16, sp()) == 0
+                assert lib.msd_layernorm(xp, yp, g, b, r, d, 1e-5, F16, sp()) == 0
+
+        def add_ln_fused():
+            for x, res, y in zip(xs, rs, ys):
+                xp, rp, yp = vp(x.data_ptr()), vp(res.data_ptr()), vp(y.data_ptr())
+                assert lib.msd_add_layernorm(xp, rp, xp, yp, g, b, r, d, 1e-5, F16, sp()) == 0
+
+        t = measure({"l2": add_then_ln, "l1": add_ln_fused}, copies)
+        rows.append({"what": "elemwise_add + LayerNorm (transformer block)", "shape": {"rows": r, "dim": d},
+                     "us_separate": round(t["l2"], 2), "us_fused": round(t["l1"], 2),
+                     "speedup": round(t["l2"] / t["l1"], 2)})
+        del xs, rs, ys
+    torch.cuda.empty_cache()
+    return rows
+
+
 def cpu_baseline(total_bytes, budget_s=12.0):
     """The reference path as host loops (the CPU oracle, fp32, unfused passes exactly as the
     reference enqueues them) over the layers of one full step, timed on this host's cores.
@@ -432,6 +524,7 @@ def main():
     }
     if not args.no_shapes:
         out["shapes"] = shape_table(torch, msd, dev, stream)
+        out["fusions"] = fusion_table(torch, msd, dev, stream)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(step.bytes)
     else:

@@ -81,6 +81,26 @@ int msd_groupnorm(const void *x, void *y, const float *gamma, const float *beta,
                   int fuse_silu, int dtype, void *stream);
 
 /*
+ * GroupNorm whose result is stored token-major: x is [batch, channels, hw], y is
+ * [batch, hw, channels], y[b, p, c] = GroupNorm(x)[b, c, p].  Replaces GroupNorm::forward
+ * followed by the permute3D_0_2_1 enqueue of SpatialTransformer::forward
+ * (M/nn/SpatialTransformer.cpp:127-139; K/util.cl:47-64) in one launch; equal to
+ * msd_groupnorm + that permute up to the summation order of the statistics (a few float
+ * ulps).  No SiLU (the reference has none there; its eps is 1e-6).  y must not overlap x.
+ */
+int msd_groupnorm_tokens(const void *x, void *y, const float *gamma, const float *beta, size_t batch,
+                         size_t channels, size_t hw, size_t groups, float eps, int dtype,
+                         void *stream);
+
+/*
+ * dst[i, k, j] = src[i, j, k]: the permute3D_0_2_1 kernel (K/util.cl:47-64) that
+ * SpatialTransformer::forward enqueues between NCHW and token layout
+ * (M/nn/SpatialTransformer.cpp:132-139,157-164).  dst must not overlap src.
+ */
+int msd_permute_0_2_1(const void *src, void *dst, size_t isize, size_t jsize, size_t ksize, int dtype,
+                      void *stream);
+
+/*
  * LayerNorm over the last dimension of a row-major [rows, dim] tensor.
  * Replaces LayerNorm::forward (M/nn/LayerNorm.cpp:94-139; K/layer_norm.cl:1-78);
  * the reference's eps is the constant 1e-5 (K/layer_norm.cl:58).  y may alias x.

@@ -25,6 +25,7 @@ C_ABI_SYMBOLS = (
     "msd_set_tuning", "msd_groupnorm", "msd_layernorm", "msd_geglu",
     "msd_silu", "msd_gelu", "msd_quick_gelu", "msd_timestep_embedding", "msd_ddim_timesteps",
     "msd_elemwise_add", "msd_chunkwise_add", "msd_chunk_add_groupnorm", "msd_add_layernorm", "msd_copy",
+    "msd_groupnorm_tokens", "msd_permute_0_2_1",
 )
 
 _lib = None
@@ -57,6 +58,8 @@ def load_library(path=None):
     lib.msd_layernorm.argtypes = [vp, vp, vp, vp, sz, sz, fl, it, vp]
     lib.msd_geglu.argtypes = [vp, vp, sz, sz, it, vp]
     lib.msd_copy.argtypes = [vp, vp, sz, vp]
+    lib.msd_permute_0_2_1.argtypes = [vp, vp, sz, sz, sz, it, vp]
+    lib.msd_groupnorm_tokens.argtypes = [vp, vp, vp, vp, sz, sz, sz, sz, fl, it, vp]
     lib.msd_elemwise_add.argtypes = [vp, vp, vp, sz, it, vp]
     lib.msd_chunkwise_add.argtypes = [vp, vp, vp, sz, sz, it, vp]
     lib.msd_chunk_add_groupnorm.argtypes = [vp, vp, vp, vp, vp, sz, sz, sz, sz, fl, it, it, vp]
@@ -114,6 +117,26 @@ def groupnorm(x, gamma, beta, groups, eps=1e-5, fuse_silu=False, out=None):
     hw = x.numel() // (batch * channels) if batch * channels else 0
     check(load_library().msd_groupnorm(_dev(x), _dev(out), _dev(gamma), _dev(beta), batch, channels,
                                        hw, groups, eps, int(fuse_silu), _dtype_code(x), _stream()))
+    return out
+
+
+def groupnorm_tokens(x, gamma, beta, groups, eps=1e-6):
+    """x: [batch, C, ...] -> [batch, H*W, C] = GroupNorm(x) with channels last (no SiLU)."""
+    import torch
+    batch, channels = x.shape[0], x.shape[1]
+    hw = x.numel() // (batch * channels) if batch * channels else 0
+    out = torch.empty((batch, hw, channels), dtype=x.dtype, device=x.device)
+    check(load_library().msd_groupnorm_tokens(_dev(x), _dev(out), _dev(gamma), _dev(beta), batch, channels,
+                                              hw, groups, eps, _dtype_code(x), _stream()))
+    return out
+
+
+def permute_0_2_1(x):
+    """[i, j, k] -> [i, k, j] (new tensor)."""
+    import torch
+    i, j, k = x.shape
+    out = torch.empty((i, k, j), dtype=x.dtype, device=x.device)
+    check(load_library().msd_permute_0_2_1(_dev(x), _dev(out), i, j, k, _dtype_code(x), _stream()))
     return out
 
 

@@ -180,6 +180,18 @@ int msd_chunk_add_groupnorm(const void *x, const void *chunk, void *y, const flo
                            dtype, stream);
 }
 
+int msd_groupnorm_tokens(const void *x, void *y, const float *gamma, const float *beta, size_t batch,
+                         size_t channels, size_t hw, size_t groups, float eps, int dtype,
+                         void *stream) {
+    if (groups == 0 || channels == 0 || channels % groups != 0) return MSD_ERR_INVALID_VALUE;
+    if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
+    if (batch * hw != 0 && (!x || !y || !gamma || !beta || x == y)) return MSD_ERR_INVALID_VALUE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == MSD_DTYPE_F32)
+        return gn_tokens_dispatch<float>(x, y, gamma, beta, batch, channels, hw, groups, eps, s);
+    return gn_tokens_dispatch<__half>(x, y, gamma, beta, batch, channels, hw, groups, eps, s);
+}
+
 static int layernorm_entry(const void *x, const void *res, void *sum, void *y, const float *gamma,
                            const float *beta, size_t rows, size_t dim, float eps, int dtype,
                            void *stream) {
@@ -245,6 +257,15 @@ int msd_gelu(const void *x, void *y, size_t n, int dtype, void *stream) {
 }
 int msd_quick_gelu(const void *x, void *y, size_t n, int dtype, void *stream) {
     return act_entry(Act::QuickGelu, x, y, n, dtype, stream);
+}
+
+int msd_permute_0_2_1(const void *src, void *dst, size_t isize, size_t jsize, size_t ksize, int dtype,
+                      void *stream) {
+    if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
+    if (isize * jsize * ksize != 0 && (!src || !dst || src == dst)) return MSD_ERR_INVALID_VALUE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == MSD_DTYPE_F32) return permute_021_dispatch<float>(src, dst, isize, jsize, ksize, s);
+    return permute_021_dispatch<__half>(src, dst, isize, jsize, ksize, s);
 }
 
 int msd_copy(const void *src, void *dst, size_t bytes, void *stream) {

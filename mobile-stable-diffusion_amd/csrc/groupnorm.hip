@@ -56,6 +56,64 @@ __device__ __forceinline__ unsigned long long tagged(uint32_t tag, float v) {
     return ((unsigned long long)tag << 32) | (unsigned long long)__float_as_uint(v);
 }
 
+// Merges the slices of one unit.  Called by every lane of the workgroup with the slice's
+// (mean, M2); `epoch` is the unit's launch count as lane 0 read it at kernel start.  On return
+// stats[0] = mean and stats[1] = 1/sqrt(var + eps) of the whole unit, in LDS, after a barrier.
+// Slice l covers vectors [l * vec_per_slice, min(vec_per_unit, (l + 1) * vec_per_slice)).
+template <int EPV>
+__device__ __forceinline__ void gn_exchange(const GnScratch &scratch, const GnParams &p, uint32_t unit,
+                                            uint32_t slice, uint32_t epoch, float slice_mean,
+                                            float slice_m2, float *stats) {
+    const uint32_t tid = threadIdx.x;
+    unsigned long long *slot_mean = scratch.slot_mean + (size_t)unit * kGnMaxSplit;
+    unsigned long long *slot_m2 = scratch.slot_m2 + (size_t)unit * kGnMaxSplit;
+    if (tid < kWave) {  // wavefront 0 owns the exchange; lane 0 holds the epoch
+        const uint32_t tag = (uint32_t)__builtin_amdgcn_readfirstlane((int)epoch) + 1u;
+        if (tid == 0) {
+            __hip_atomic_store(slot_mean + slice, tagged(tag, slice_mean), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(slot_m2 + slice, tagged(tag, slice_m2), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        }
+        // lane l waits for slice l
+        float m_l = 0.0f, q_l = 0.0f, n_l = 0.0f;
+        if (tid < p.split) {
+            unsigned long long wm, wq;
+            uint32_t polls = 0;
+            bool ok;
+            do {
+                wm = __hip_atomic_load(slot_mean + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                wq = __hip_atomic_load(slot_m2 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                ok = (uint32_t)(wm >> 32) == tag && (uint32_t)(wq >> 32) == tag;
+                if (!ok) __builtin_amdgcn_s_sleep(1);
+            } while (!ok && ++polls < kGnSpinLimit);
+            if (!ok)
+                __hip_atomic_fetch_or(scratch.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            m_l = __uint_as_float((uint32_t)wm);
+            q_l = __uint_as_float((uint32_t)wq);
+            const uint32_t b = tid * p.vec_per_slice;
+            const uint32_t e = min(p.vec_per_unit, b + p.vec_per_slice);
+            n_l = (float)((e - b) * EPV);
+        }
+        // Chan: mean = sum n_l mean_l / n ; M2 = sum M2_l + sum n_l (mean_l - mean)^2
+        const float total_mean = wave_sum(m_l * n_l) * p.inv_count;
+        const float dm = m_l - total_mean;
+        const float m2 = wave_sum(fmaf(n_l * dm, dm, q_l));
+        if (tid == 0) {
+            stats[0] = total_mean;
+            stats[1] = __builtin_amdgcn_rsqf(m2 * p.inv_count + p.eps);
+            // this slice has consumed its siblings' words; the last one closes the launch
+            const uint32_t old = __hip_atomic_fetch_add(scratch.done + unit, 1u, __ATOMIC_RELAXED,
+                                                        __HIP_MEMORY_SCOPE_AGENT);
+            if (old == p.split - 1) {
+                __hip_atomic_store(scratch.done + unit, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(scratch.epoch + unit, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+    }
+    __syncthreads();
+}
+
 // FULL: every lane owns exactly K vectors (no masking anywhere).
 template <typename T, int K, bool SILU, bool FULL>
 __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
@@ -159,59 +217,7 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
         mean = slice_mean;
         rstd = __builtin_amdgcn_rsqf(slice_m2 * p.inv_count + p.eps);
     } else {
-        unsigned long long *slot_mean = scratch.slot_mean + (size_t)unit * kGnMaxSplit;
-        unsigned long long *slot_m2 = scratch.slot_m2 + (size_t)unit * kGnMaxSplit;
-        if (tid < kWave) {  // wavefront 0 owns the exchange; lane 0 holds the epoch
-            const uint32_t tag =
-                (uint32_t)__builtin_amdgcn_readfirstlane((int)epoch) + 1u;
-            if (tid == 0) {
-                __hip_atomic_store(slot_mean + slice, tagged(tag, slice_mean), __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(slot_m2 + slice, tagged(tag, slice_m2), __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-            }
-            // lane l waits for slice l
-            float m_l = 0.0f, q_l = 0.0f, n_l = 0.0f;
-            if (tid < p.split) {
-                unsigned long long wm, wq;
-                uint32_t polls = 0;
-                bool ok;
-                do {
-                    wm = __hip_atomic_load(slot_mean + tid, __ATOMIC_RELAXED,
-                                           __HIP_MEMORY_SCOPE_AGENT);
-                    wq = __hip_atomic_load(slot_m2 + tid, __ATOMIC_RELAXED,
-                                           __HIP_MEMORY_SCOPE_AGENT);
-                    ok = (uint32_t)(wm >> 32) == tag && (uint32_t)(wq >> 32) == tag;
-                    if (!ok) __builtin_amdgcn_s_sleep(1);
-                } while (!ok && ++polls < kGnSpinLimit);
-                if (!ok)
-                    __hip_atomic_fetch_or(scratch.status, 1u, __ATOMIC_RELAXED,
-                                          __HIP_MEMORY_SCOPE_AGENT);
-                m_l = __uint_as_float((uint32_t)wm);
-                q_l = __uint_as_float((uint32_t)wq);
-                const uint32_t b = tid * p.vec_per_slice;
-                const uint32_t e = min(p.vec_per_unit, b + p.vec_per_slice);
-                n_l = (float)((e - b) * EPV);
-            }
-            // Chan: mean = sum n_l mean_l / n ; M2 = sum M2_l + sum n_l (mean_l - mean)^2
-            const float total_mean = wave_sum(m_l * n_l) * p.inv_count;
-            const float dm = m_l - total_mean;
-            const float m2 = wave_sum(fmaf(n_l * dm, dm, q_l));
-            if (tid == 0) {
-                stats[0] = total_mean;
-                stats[1] = __builtin_amdgcn_rsqf(m2 * p.inv_count + p.eps);
-                // this slice has consumed its siblings' words; the last one closes the launch
-                const uint32_t old = __hip_atomic_fetch_add(scratch.done + unit, 1u, __ATOMIC_RELAXED,
-                                                            __HIP_MEMORY_SCOPE_AGENT);
-                if (old == p.split - 1) {
-                    __hip_atomic_store(scratch.done + unit, 0u, __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
-                    __hip_atomic_store(scratch.epoch + unit, tag, __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
-                }
-            }
-        }
-        __syncthreads();
+        gn_exchange<EPV>(scratch, p, unit, slice, epoch, slice_mean, slice_m2, stats);
         mean = stats[0];
         rstd = stats[1];
     }
@@ -294,6 +300,168 @@ __global__ __launch_bounds__(kGenericThreads) void gn_generic_kernel(
         const uint32_t c = ch0 + i / hw;
         const float t = fmaf(value(i) - mean, rstd * gamma[c], beta[c]);
         Store<T>::store1(yout + i, SILU ? silu_f(t) : t);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// GroupNorm with a token-major store: y[b, p, c] = GroupNorm(x)[b, c, p].
+// Replaces GroupNorm followed by the (0, 2, 1) permute that turns NCHW into tokens.
+// A slice is all channels of the group over a range of positions, so that for each position
+// the slice owns one contiguous run of ch_per_group outputs; normalised values go through
+// LDS ([channel][position], 16-byte padded pitch) and leave as 4-byte stores that walk those
+// runs.  Statistics and the exchange between slices are those of gn_slice_kernel.
+// ---------------------------------------------------------------------------
+struct GnTokParams {
+    GnParams base;        // vec_per_slice = ch_per_group * pos_vecs.d ; vec_per_unit = that * split
+    FastDiv pos_vecs;     // position vectors per slice (hw_vec / split)
+    FastDiv row_dwords;   // 4-byte words per output run: ch_per_group * sizeof(T) / 4
+    uint32_t hw;          // positions per sample
+    uint32_t channels;
+    uint32_t pitch;       // LDS elements between channels: positions per slice + 16 bytes
+};
+
+template <typename T, int K>
+__global__ __launch_bounds__(kGnMaxThreads) void gn_tokens_kernel(
+    const T *__restrict__ x, T *__restrict__ y, const float *__restrict__ gamma,
+    const float *__restrict__ beta, GnScratch scratch, GnTokParams q) {
+    constexpr int EPV = Store<T>::EPV;
+    extern __shared__ u32x4 lds_vec[];
+    __shared__ float red_a[kGnMaxThreads / kWave];
+    __shared__ float red_b[kGnMaxThreads / kWave];
+    __shared__ float stats[2];
+    const GnParams &p = q.base;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t nt = blockDim.x;
+    const uint32_t unit = blockIdx.x >> p.split_shift;
+    const uint32_t slice = blockIdx.x & (p.split - 1);
+    const uint32_t nvec = p.vec_per_slice;
+    const uint32_t pvs = q.pos_vecs.d;
+    const u32x4 *xin = reinterpret_cast<const u32x4 *>(x) + (size_t)unit * p.vec_per_unit;
+
+    uint32_t epoch = 0;
+    if (p.split > 1 && tid == 0)
+        epoch = __hip_atomic_load(scratch.epoch + unit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+    // lane-local vector -> (channel of the group, position vector of the slice)
+    u32x4 raw[K];
+    uint32_t cl[K], pv[K];
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        const uint32_t vl = min(k * nt + tid, nvec - 1);  // ragged tail re-reads the last vector
+        cl[k] = fast_div(vl, q.pos_vecs);
+        pv[k] = vl - cl[k] * pvs;
+        raw[k] = load_stream(xin + (size_t)cl[k] * p.hw_vec.d + slice * pvs + pv[k]);
+    }
+    const uint32_t ch0 = (unit % p.groups) * p.ch_per_group;
+
+    float s = 0.0f;
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        float f[EPV];
+        Store<T>::unpack(raw[k], f);
+        float sk = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EPV; e++) sk += f[e];
+        s += (k * nt + tid < nvec) ? sk : 0.0f;
+    }
+    const float slice_mean = block_sum_rt(s, red_a) / (float)(nvec * EPV);
+    if (sizeof(T) == 2) {
+#pragma unroll
+        for (int k = 0; k < K; k++) forget(raw[k]);
+    }
+    float m2 = 0.0f;
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        float f[EPV];
+        Store<T>::unpack(raw[k], f);
+        float qk = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EPV; e++) {
+            const float d = f[e] - slice_mean;
+            qk = fmaf(d, d, qk);
+        }
+        m2 += (k * nt + tid < nvec) ? qk : 0.0f;
+    }
+    const float slice_m2 = block_sum_rt(m2, red_b);
+    if (sizeof(T) == 2) {
+#pragma unroll
+        for (int k = 0; k < K; k++) forget(raw[k]);
+    }
+
+    float mean, rstd;
+    if (p.split == 1) {
+        mean = slice_mean;
+        rstd = __builtin_amdgcn_rsqf(slice_m2 * p.inv_count + p.eps);
+    } else {
+        gn_exchange<EPV>(scratch, p, unit, slice, epoch, slice_mean, slice_m2, stats);
+        mean = stats[0];
+        rstd = stats[1];
+    }
+
+    // ---- normalise into LDS as [channel][position]
+    T *lds = reinterpret_cast<T *>(lds_vec);
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        if (k * nt + tid < nvec) {
+            const float a = rstd * gamma[ch0 + cl[k]];
+            const float b = beta[ch0 + cl[k]];
+            float f[EPV];
+            Store<T>::unpack(raw[k], f);
+#pragma unroll
+            for (int e = 0; e < EPV; e++) f[e] = fmaf(f[e] - mean, a, b);
+            *reinterpret_cast<u32x4 *>(lds + (size_t)cl[k] * q.pitch + pv[k] * EPV) = Store<T>::pack(f);
+        }
+    }
+    __syncthreads();
+
+    // ---- token-major store: for each position of the slice one run of ch_per_group values
+    const uint32_t rows = pvs * EPV;                         // positions in the slice
+    const uint32_t words = rows * q.row_dwords.d;            // 4-byte words to write
+    const uint32_t sample = unit / p.groups;
+    const size_t first = ((size_t)sample * q.hw + (size_t)slice * rows) * q.channels + ch0;
+    uint32_t *out = reinterpret_cast<uint32_t *>(y + first);
+    const uint32_t row_stride = q.channels * sizeof(T) / 4;  // words between positions
+    for (uint32_t i = tid; i < words; i += nt) {
+        const uint32_t r = fast_div(i, q.row_dwords);
+        const uint32_t c = i - r * q.row_dwords.d;
+        uint32_t w;
+        if (sizeof(T) == 2) {
+            const uint16_t lo = reinterpret_cast<const uint16_t *>(lds)[(2 * c) * q.pitch + r];
+            const uint16_t hi = reinterpret_cast<const uint16_t *>(lds)[(2 * c + 1) * q.pitch + r];
+            w = (uint32_t)lo | ((uint32_t)hi << 16);
+        } else {
+            w = reinterpret_cast<const uint32_t *>(lds)[c * q.pitch + r];
+        }
+        out[(size_t)r * row_stride + c] = w;
+    }
+}
+
+// Any shape: one workgroup per unit, three passes, element-wise scattered stores.
+template <typename T>
+__global__ __launch_bounds__(kGenericThreads) void gn_tokens_generic_kernel(
+    const T *__restrict__ x, T *__restrict__ y, const float *__restrict__ gamma,
+    const float *__restrict__ beta, uint32_t unit_size, uint32_t hw, uint32_t groups,
+    uint32_t ch_per_group, float eps) {
+    __shared__ float red_a[kGenericThreads / kWave];
+    __shared__ float red_b[kGenericThreads / kWave];
+    const uint32_t unit = blockIdx.x;
+    const T *xin = x + (size_t)unit * unit_size;
+    float s = 0.0f;
+    for (uint32_t i = threadIdx.x; i < unit_size; i += kGenericThreads) s += Store<T>::load1(xin + i);
+    const float mean = block_sum_rt(s, red_a) / (float)unit_size;
+    float m2 = 0.0f;
+    for (uint32_t i = threadIdx.x; i < unit_size; i += kGenericThreads) {
+        const float d = Store<T>::load1(xin + i) - mean;
+        m2 = fmaf(d, d, m2);
+    }
+    const float rstd = 1.0f / sqrtf(block_sum_rt(m2, red_b) / (float)unit_size + eps);
+    const uint32_t ch0 = (unit % groups) * ch_per_group;
+    const uint32_t channels = groups * ch_per_group;
+    T *yout = y + (size_t)(unit / groups) * hw * channels;
+    for (uint32_t i = threadIdx.x; i < unit_size; i += kGenericThreads) {
+        const uint32_t c = ch0 + i / hw, pos = i % hw;
+        const float t = fmaf(Store<T>::load1(xin + i) - mean, rstd * gamma[c], beta[c]);
+        Store<T>::store1(yout + (size_t)pos * channels + c, t);
     }
 }
 
@@ -461,5 +629,104 @@ template int gn_dispatch<float>(const void *, const void *, void *, const float 
                                 size_t, size_t, size_t, size_t, float, bool, hipStream_t);
 template int gn_dispatch<__half>(const void *, const void *, void *, const float *, const float *,
                                  size_t, size_t, size_t, size_t, float, bool, hipStream_t);
+
+namespace {
+
+template <typename T, int K>
+void gn_tokens_launch(uint32_t blocks, uint32_t threads, size_t lds_bytes, hipStream_t stream,
+                      const T *x, T *y, const float *gamma, const float *beta, const GnScratch &sc,
+                      const GnTokParams &q) {
+    hipLaunchKernelGGL((gn_tokens_kernel<T, K>), dim3(blocks), dim3(threads), lds_bytes, stream, x, y,
+                       gamma, beta, sc, q);
+}
+
+}  // namespace
+
+template <typename T>
+int gn_tokens_dispatch(const void *xv, void *yv, const float *gamma, const float *beta, size_t batch,
+                       size_t channels, size_t hw, size_t groups, float eps, hipStream_t stream) {
+    constexpr int EPV = Store<T>::EPV;
+    constexpr uint32_t kMaxK = sizeof(T) == 4 ? 10 : kGnMaxK;
+    constexpr size_t kMaxLds = 60 * 1024;
+    const T *x = static_cast<const T *>(xv);
+    T *y = static_cast<T *>(yv);
+    const size_t cpg = channels / groups;
+    const size_t unit_size = cpg * hw;
+    const size_t units = batch * groups;
+    if (units == 0 || unit_size == 0) return MSD_OK;
+    if (units > 0x7FFFFFFFull || unit_size > 0x7FFFFFFFull) return MSD_ERR_INVALID_VALUE;
+    auto generic = [&]() {
+        hipLaunchKernelGGL((gn_tokens_generic_kernel<T>), dim3((uint32_t)units), dim3(kGenericThreads), 0,
+                           stream, x, y, gamma, beta, (uint32_t)unit_size, (uint32_t)hw, (uint32_t)groups,
+                           (uint32_t)cpg, eps);
+        return launch_status();
+    };
+    const bool vector_ok = aligned16(x) && (reinterpret_cast<uintptr_t>(y) & 3u) == 0 && hw % EPV == 0 &&
+                           (cpg * sizeof(T)) % 4 == 0 && (channels * sizeof(T)) % 4 == 0;
+    if (!vector_ok) return generic();
+    const size_t hw_vec = hw / EPV;
+    // slices cut the positions: the split must divide them, fit the registers and the LDS
+    uint32_t want = 1;
+    if (unit_size > 24576) {
+        want = 4;
+        if (units * 4 < 192 && unit_size >= 65536) want = 8;
+    }
+    if (g_tuning.gn_split > 0) want = (uint32_t)g_tuning.gn_split;
+    uint32_t split = 0;
+    for (uint32_t s = 1; s <= kGnMaxSplit; s *= 2) {
+        if (hw_vec % s != 0) break;
+        const size_t nvec = cpg * (hw_vec / s);
+        const size_t lds = cpg * (hw / s + 16 / sizeof(T)) * sizeof(T);
+        if (nvec > (size_t)kGnMaxThreads * kMaxK || lds > kMaxLds) continue;
+        split = s;
+        if (s >= want) break;
+    }
+    if (split == 0 || (split > 1 && units > kGnMaxUnits)) return generic();
+
+    GnTokParams q;
+    const size_t pvs = hw_vec / split;
+    const size_t nvec = cpg * pvs;
+    q.base.vec_per_unit = (uint32_t)(nvec * split);
+    q.base.vec_per_slice = (uint32_t)nvec;
+    q.base.split = split;
+    q.base.split_shift = (uint32_t)__builtin_ctz(split);
+    q.base.groups = (uint32_t)groups;
+    q.base.ch_per_group = (uint32_t)cpg;
+    q.base.hw_vec = make_fast_div((uint32_t)hw_vec);
+    q.base.eps = eps;
+    q.base.inv_count = 1.0f / (float)unit_size;
+    q.pos_vecs = make_fast_div((uint32_t)pvs);
+    q.row_dwords = make_fast_div((uint32_t)(cpg * sizeof(T) / 4));
+    q.hw = (uint32_t)hw;
+    q.channels = (uint32_t)channels;
+    q.pitch = (uint32_t)(pvs * EPV + 16 / sizeof(T));
+    const size_t lds_bytes = cpg * q.pitch * sizeof(T);
+    const GnPlan pl = plan_slice((uint32_t)nvec, split, 0, kMaxK);
+    if (pl.k == 0) return generic();
+    GnScratch sc{nullptr, nullptr, nullptr, nullptr, nullptr};
+    if (split > 1) {
+        const hipError_t err = get_scratch(stream, &sc);
+        if (err != hipSuccess) return (int)err;
+    }
+    const uint32_t blocks = (uint32_t)(units * split);
+    switch (pl.k) {
+        case 1: gn_tokens_launch<T, 1>(blocks, pl.threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
+        case 2: gn_tokens_launch<T, 2>(blocks, pl.threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
+        case 3: gn_tokens_launch<T, 3>(blocks, pl.threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
+        case 4: gn_tokens_launch<T, 4>(blocks, pl.threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
+        case 5: gn_tokens_launch<T, 5>(blocks, pl.threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
+        case 6: gn_tokens_launch<T, 6>(blocks, pl.threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
+        case 8: gn_tokens_launch<T, 8>(blocks, pl.threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
+        case 10: gn_tokens_launch<T, 10>(blocks, pl.threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
+        case 12: gn_tokens_launch<T, 12>(blocks, pl.threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
+        default: gn_tokens_launch<T, 16>(blocks, pl.threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
+    }
+    return launch_status();
+}
+
+template int gn_tokens_dispatch<float>(const void *, void *, const float *, const float *, size_t, size_t,
+                                       size_t, size_t, float, hipStream_t);
+template int gn_tokens_dispatch<__half>(const void *, void *, const float *, const float *, size_t, size_t,
+                                        size_t, size_t, float, hipStream_t);
 
 }  // namespace msd

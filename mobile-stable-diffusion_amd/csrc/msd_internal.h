@@ -43,6 +43,10 @@ template <typename T>
 int gn_dispatch(const void *x, const void *chunk, void *y, const float *gamma, const float *beta,
                 size_t batch, size_t channels, size_t hw, size_t groups, float eps, bool silu,
                 hipStream_t stream);
+// y is token-major [batch, hw, channels]; must not overlap x
+template <typename T>
+int gn_tokens_dispatch(const void *x, void *y, const float *gamma, const float *beta, size_t batch,
+                       size_t channels, size_t hw, size_t groups, float eps, hipStream_t stream);
 // res / sum may be null (plain LayerNorm); otherwise sum = x + res is written and normalised
 template <typename T>
 int ln_dispatch(const void *x, const void *res, void *sum, void *y, const float *gamma,
@@ -52,6 +56,10 @@ int add_dispatch(const void *a, const void *b, void *c, size_t n, size_t chunk_s
                  hipStream_t stream);  // chunk_size 0: elementwise; else b holds one value per chunk
 template <typename T>
 int geglu_dispatch(const void *proj, void *out, size_t rows, size_t inner, hipStream_t stream);
+
+template <typename T>
+int permute_021_dispatch(const void *src, void *dst, size_t isize, size_t jsize, size_t ksize,
+                         hipStream_t stream);
 
 enum class Act { Silu, Gelu, QuickGelu, Copy };
 template <typename T>

@@ -6,6 +6,7 @@
 #include "msd_internal.h"
 
 #include <cmath>
+#include <type_traits>
 
 namespace msd {
 namespace {
@@ -150,6 +151,55 @@ __global__ __launch_bounds__(kStreamThreads) void add_generic_kernel(const T *a,
 }
 
 // ---------------------------------------------------------------------------
+// [i, j, k] -> [i, k, j] through a 64 x 64 LDS tile: reads run along k, writes along j, both in
+// 4-element pieces (8 or 16 bytes), tile rows padded by one piece against bank conflicts.
+// ---------------------------------------------------------------------------
+constexpr int kTile = 64;
+
+template <typename T>
+__global__ __launch_bounds__(256) void permute_021_kernel(const T *__restrict__ src,
+                                                          T *__restrict__ dst, uint32_t jsize,
+                                                          uint32_t ksize) {
+    typedef T vec4 __attribute__((ext_vector_type(4)));
+    __shared__ T tile[kTile][kTile + 4];
+    const uint32_t k0 = blockIdx.x * kTile, j0 = blockIdx.y * kTile, i = blockIdx.z;
+    const T *in = src + (size_t)i * jsize * ksize;
+    T *out = dst + (size_t)i * jsize * ksize;
+    const uint32_t lane4 = (threadIdx.x & 15) * 4, row = threadIdx.x >> 4;  // 16 rows per pass
+#pragma unroll
+    for (int pass = 0; pass < 4; pass++) {
+        const uint32_t j = j0 + row + pass * 16, k = k0 + lane4;
+        if (j < jsize && k < ksize) {  // jsize, ksize are multiples of 4: a piece is all in or out
+            const vec4 v = *reinterpret_cast<const vec4 *>(in + (size_t)j * ksize + k);
+#pragma unroll
+            for (int e = 0; e < 4; e++) tile[row + pass * 16][lane4 + e] = v[e];
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int pass = 0; pass < 4; pass++) {
+        const uint32_t k = k0 + row + pass * 16, j = j0 + lane4;
+        if (k < ksize && j < jsize) {
+            vec4 v;
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = tile[lane4 + e][row + pass * 16];
+            *reinterpret_cast<vec4 *>(out + (size_t)k * jsize + j) = v;
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kStreamThreads) void permute_021_generic_kernel(
+    const T *__restrict__ src, T *__restrict__ dst, size_t isize, size_t jsize, size_t ksize) {
+    const size_t n = isize * jsize * ksize;
+    for (size_t d = (size_t)blockIdx.x * kStreamThreads + threadIdx.x; d < n;
+         d += (size_t)gridDim.x * kStreamThreads) {
+        const size_t j = d % jsize, k = (d / jsize) % ksize, i = d / (jsize * ksize);
+        dst[d] = src[(i * jsize + j) * ksize + k];
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Timestep embedding
 // ---------------------------------------------------------------------------
 // freq_i is the float32 expression exp(neg_log_period * float(i) / float(half))
@@ -269,6 +319,31 @@ int add_dispatch(const void *av, const void *bv, void *cv, size_t n, size_t chun
     return launch_status();
 }
 
+template <typename TT>
+int permute_021_dispatch(const void *srcv, void *dstv, size_t isize, size_t jsize, size_t ksize,
+                         hipStream_t stream) {
+    // pure data movement: elements are handled as raw 16- or 32-bit words
+    typedef typename std::conditional<sizeof(TT) == 2, uint16_t, uint32_t>::type T;
+    const T *src = static_cast<const T *>(srcv);
+    T *dst = static_cast<T *>(dstv);
+    if (isize * jsize * ksize == 0) return MSD_OK;
+    const uintptr_t piece = 4 * sizeof(T);
+    const bool tiled = jsize % 4 == 0 && ksize % 4 == 0 && reinterpret_cast<uintptr_t>(src) % piece == 0 &&
+                       reinterpret_cast<uintptr_t>(dst) % piece == 0 && isize <= 65535 &&
+                       (jsize + kTile - 1) / kTile <= 65535 && ksize < 0x7FFFFFFFull && jsize < 0x7FFFFFFFull;
+    if (tiled) {
+        hipLaunchKernelGGL((permute_021_kernel<T>),
+                           dim3((uint32_t)((ksize + kTile - 1) / kTile), (uint32_t)((jsize + kTile - 1) / kTile),
+                                (uint32_t)isize),
+                           dim3(256), 0, stream, src, dst, (uint32_t)jsize, (uint32_t)ksize);
+    } else {
+        const size_t want = (isize * jsize * ksize + kStreamThreads - 1) / kStreamThreads;
+        hipLaunchKernelGGL((permute_021_generic_kernel<T>), dim3((uint32_t)(want < 65536 ? want : 65536)),
+                           dim3(kStreamThreads), 0, stream, src, dst, isize, jsize, ksize);
+    }
+    return launch_status();
+}
+
 template <typename T>
 int act_dispatch(Act op, const void *x, void *y, size_t n, hipStream_t stream) {
     switch (op) {
@@ -295,6 +370,8 @@ template int geglu_dispatch<float>(const void *, void *, size_t, size_t, hipStre
 template int geglu_dispatch<__half>(const void *, void *, size_t, size_t, hipStream_t);
 template int add_dispatch<float>(const void *, const void *, void *, size_t, size_t, hipStream_t);
 template int add_dispatch<__half>(const void *, const void *, void *, size_t, size_t, hipStream_t);
+template int permute_021_dispatch<float>(const void *, void *, size_t, size_t, size_t, hipStream_t);
+template int permute_021_dispatch<__half>(const void *, void *, size_t, size_t, size_t, hipStream_t);
 template int act_dispatch<float>(Act, const void *, void *, size_t, hipStream_t);
 template int act_dispatch<__half>(Act, const void *, void *, size_t, hipStream_t);
 template int temb_dispatch<float>(const int64_t *, void *, size_t, size_t, float, hipStream_t);

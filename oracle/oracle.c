@@ -264,6 +264,14 @@ void orc_chunkwise_add(const float *a, const float *chunk, float *c, size_t n, s
     for (size_t i = 0; i < n; i++) c[i] = a[i] + chunk[i / chunk_size]; /* K/util.cl:143-147 */
 }
 
+void orc_permute3D_0_2_1(const float *src, float *dst, size_t isize, size_t jsize, size_t ksize) {
+    /* K/util.cl:47-64: i j k -> i k j */
+    for (size_t i = 0; i < isize; i++)
+        for (size_t j = 0; j < jsize; j++)
+            for (size_t k = 0; k < ksize; k++)
+                dst[i * ksize * jsize + k * jsize + j] = src[i * jsize * ksize + j * ksize + k];
+}
+
 void orc_timestep_freqs(float *freq, int half, float max_period) {
     for (int i = 0; i < half; i++) /* M/UNetModel.cpp:1950, float overloads throughout */
         freq[i] = expf((-logf(max_period)) * (float)i / (float)half);

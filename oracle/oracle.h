@@ -22,8 +22,8 @@
  *        cross-check, torch float32 fixture of the textbook formula.
  *   orc_ddim_timesteps : closed form 1+c*k and the reference's shipped
  *        literal 981 (native-lib.cpp:240) as the first step of 50.
- *   orc_elemwise_add, orc_chunkwise_add : exact float additions; checked against numpy
- *        broadcasting (bit-exact).
+ *   orc_elemwise_add, orc_chunkwise_add, orc_permute3D_0_2_1 : exact; checked against numpy
+ *        broadcasting / transpose (bit-exact).
  *   orc_quick_gelu : PARITY UNPINNED BY THE REFERENCE (the reference has no
  *        quick_GELU); pinned only by the closed form x*sigmoid(1.702x).
  */
@@ -75,6 +75,8 @@ void orc_quick_gelu(const float *src, float *dst, size_t n);
 void orc_elemwise_add(const float *a, const float *b, float *c, size_t n);
 /* K/util.cl:136-148: c[i] = a[i] + chunk[i / chunk_size] */
 void orc_chunkwise_add(const float *a, const float *chunk, float *c, size_t n, size_t chunk_size);
+/* K/util.cl:47-64: [i, j, k] -> [i, k, j] */
+void orc_permute3D_0_2_1(const float *src, float *dst, size_t isize, size_t jsize, size_t ksize);
 /* K/geglu.cl:1-25: value = first half of a row, gate = second half */
 void orc_gelu_multiply(const float *ab, float *dst, size_t rows, size_t inner);
 /* M/UNetModel.cpp:1935-1958 */

@@ -56,6 +56,7 @@ def lib():
         "orc_gelu_multiply": (None, [_f32p, _f32p, _sz, _sz]),
         "orc_elemwise_add": (None, [_f32p, _f32p, _f32p, _sz]),
         "orc_chunkwise_add": (None, [_f32p, _f32p, _f32p, _sz, _sz]),
+        "orc_permute3D_0_2_1": (None, [_f32p, _f32p, _sz, _sz, _sz]),
         "orc_timestep_embedding": (None, [_i64, _f32p, _it, _fl]),
         "orc_timestep_freqs": (None, [_f32p, _it, _fl]),
         "orc_ddim_timesteps": (_it, [_it, _i32p, _it]),
@@ -189,6 +190,15 @@ def chunkwise_add(a, chunk, chunk_size):
     c = np.empty_like(a)
     lib().orc_chunkwise_add(a.reshape(-1), _c(chunk), c.reshape(-1), a.size, chunk_size)
     return c
+
+
+def permute_0_2_1(x):
+    """[i, j, k] -> [i, k, j]."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    i, j, k = x.shape
+    y = np.empty((i, k, j), dtype=np.float32)
+    lib().orc_permute3D_0_2_1(x.reshape(-1), y.reshape(-1), i, j, k)
+    return y
 
 
 def timestep_embedding(t, dim=320, max_period=10000.0):

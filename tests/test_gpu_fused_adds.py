@@ -2,6 +2,8 @@
 ResBlock out-norm, elemwise_add before LayerNorm 2 / 3) and their fusion into the norm
 kernels.  Fused launches must equal the two-launch sequence bit for bit, and both must match
 the CPU oracle's restatement of the reference kernels."""
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -102,9 +104,68 @@ def test_add_layernorm_equals_two_launches(msd, orc, cuda, rows, dim, half):
         assert_close_f32(got, ref, what="add ln f32")
 
 
+@pytest.mark.parametrize("half", [False, True], ids=["f32", "f16"])
+@pytest.mark.parametrize("shape,groups,split", [((2, 320, 64, 64), 32, 0), ((2, 640, 32, 32), 32, 0),
+                                                ((2, 1280, 16, 16), 32, 0), ((2, 1280, 8, 8), 32, 0),
+                                                ((1, 320, 64, 64), 32, 8), ((2, 640, 32, 32), 32, 2),
+                                                ((1, 96, 24, 24), 32, 0), ((3, 64, 5, 7), 8, 0),
+                                                ((1, 33, 4, 4), 33, 0), ((1, 8, 128, 128), 1, 0)])
+def test_groupnorm_tokens_equals_norm_then_permute(msd, orc, cuda, shape, groups, split, half):
+    """SpatialTransformer's GroupNorm(eps 1e-6, no SiLU) + permute (0, 2, 1) in one launch
+    (M/nn/SpatialTransformer.cpp:127-139)."""
+    import torch
+    lib = msd.load_library()
+    batch, channels = shape[0], shape[1]
+    hw = int(np.prod(shape[2:]))
+    x = orc.normal(shape, seed=sum(shape) + 3, sigma=1.5, mean=0.4)
+    g, b = _affine(orc, channels, 11)
+    xin = orc.round_to_half(x) if half else x
+    xd, gd, bd = _dev(xin, cuda, half), _dev(g, cuda), _dev(b, cuda)
+    try:
+        lib.msd_set_tuning(msd.TUNE_GN_SPLIT, split)
+        fused = msd.groupnorm_tokens(xd, gd, bd, groups, 1e-6)
+    finally:
+        lib.msd_set_tuning(msd.TUNE_GN_SPLIT, 0)
+    two = msd.groupnorm(xd, gd, bd, groups, 1e-6, False).view(batch, channels, hw).permute(0, 2, 1).contiguous()
+    assert fused.shape == (batch, hw, channels)
+    # the slices cut positions instead of channel ranges, so the statistics are summed in another
+    # order: equal to the two-launch result up to that (a few float ulps), not bit for bit
+    d = (fused.float() - two.float()).abs()
+    if half:
+        assert (d == 0).float().mean().item() > 0.999
+        assert_close_f16(fused.float().cpu().numpy(), two.float().cpu().numpy(), "gn tokens vs two launches")
+    else:
+        assert (d / two.abs().clamp(min=1.0)).max().item() < 2e-6
+    ref = np.concatenate([orc.permute_0_2_1(orc.groupnorm64(xin, g, b, groups, 1e-6, False)
+                                            .astype(np.float32).reshape(batch, channels, hw)[i:i + 1])
+                          for i in range(batch)])
+    got = fused.float().cpu().numpy()
+    if half:
+        assert_close_f16(got, orc.round_to_half(ref), "gn tokens f16")
+    else:
+        assert_close_f32(got, ref, what="gn tokens f32")
+    assert msd.status() == 0
+
+
+@pytest.mark.parametrize("half", [False, True], ids=["f32", "f16"])
+@pytest.mark.parametrize("shape", [(2, 320, 4096), (2, 4096, 320), (1, 1280, 64), (3, 100, 36), (2, 7, 5),
+                                   (1, 64, 64), (5, 68, 132), (1, 1, 8)])
+def test_permute_0_2_1(msd, orc, cuda, shape, half):
+    import torch
+    x = orc.normal(shape, seed=sum(shape))
+    xin = orc.round_to_half(x) if half else x
+    got = msd.permute_0_2_1(_dev(xin, cuda, half))
+    assert np.array_equal(got.float().cpu().numpy(), orc.permute_0_2_1(xin))
+    assert torch.equal(msd.permute_0_2_1(got), _dev(xin, cuda, half))  # its own inverse
+
+
 def test_fused_argument_checks(msd, cuda):
     lib = msd.load_library()
     assert lib.msd_chunk_add_groupnorm(None, None, None, None, None, 1, 32, 16, 32, 1e-5, 0, 0, None) == 1
     assert lib.msd_add_layernorm(None, None, None, None, None, None, 4, 64, 1e-5, 0, None) == 1
     assert lib.msd_chunkwise_add(None, None, None, 16, 0, 0, None) == 1
     assert lib.msd_elemwise_add(None, None, None, 0, 0, None) == 0
+    import torch
+    x = torch.zeros(32 * 64, device=cuda)
+    p = ctypes.c_void_p(x.data_ptr())
+    assert lib.msd_groupnorm_tokens(p, p, p, p, 1, 32, 64, 32, 1e-6, 0, None) == 1  # y must not be x

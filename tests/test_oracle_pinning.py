@@ -167,6 +167,8 @@ def test_add_kernels_are_exact(orc):
     assert np.array_equal(orc.elemwise_add(a, b), a + b)
     chunk = orc.normal((2, 6), seed=83)  # one value per (sample, channel), broadcast over H*W
     assert np.array_equal(orc.chunkwise_add(a, chunk, 35), a + chunk[:, :, None, None])
+    t = orc.normal((3, 5, 7), seed=84)
+    assert np.array_equal(orc.permute_0_2_1(t), t.transpose(0, 2, 1))
 
 
 # ----------------------------------------------------------------- timestep embedding
