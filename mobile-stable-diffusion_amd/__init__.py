@@ -270,6 +270,7 @@ def load_nn_library(path=None):
         "msdnn_groupnorm_check": (it, [vp, sz, it]),
         "msdnn_groupnorm_forward": (it, [vp, vp, vp, sz, it]),
         "msdnn_groupnorm_forward_chunk": (it, [vp, vp, vp, sz, vp, sz, it]),
+        "msdnn_groupnorm_forward_tokens": (it, [vp, vp, vp, sz, it]),
         "msdnn_groupnorm_destroy": (None, [vp]),
         "msdnn_layernorm_create": (vp, [vp, sz, cp, cp, fl]),
         "msdnn_layernorm_init": (it, [vp]),

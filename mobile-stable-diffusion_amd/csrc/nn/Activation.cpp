@@ -37,4 +37,11 @@ int chunkwise_add(hipStream_t stream, const DeviceBuffer &a, const DeviceBuffer 
     return msd_chunkwise_add(a.ptr(), chunk.ptr(), c.ptr(), a.count(), chunk_size, (int)a.dtype(), stream);
 }
 
+int permute3D_0_2_1(hipStream_t stream, const DeviceBuffer &src, DeviceBuffer &dst, size_t isize,
+                    size_t jsize, size_t ksize) {
+    if (dst.bytes() != src.bytes() || dst.dtype() != src.dtype() || src.count() != isize * jsize * ksize)
+        throw std::runtime_error("buffer size does not match i * j * k");
+    return msd_permute_0_2_1(src.ptr(), dst.ptr(), isize, jsize, ksize, (int)src.dtype(), stream);
+}
+
 }  // namespace msd

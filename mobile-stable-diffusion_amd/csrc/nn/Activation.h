@@ -22,4 +22,9 @@ int elemwise_add(hipStream_t stream, const DeviceBuffer &a, const DeviceBuffer &
 int chunkwise_add(hipStream_t stream, const DeviceBuffer &a, const DeviceBuffer &chunk, DeviceBuffer &c,
                   size_t chunk_size);
 
+// dst[i, k, j] = src[i, j, k]: utilKernel->permute3D_0_2_1 (K/util.cl:47-64), enqueued by
+// SpatialTransformer::forward with global size {i, j, k} (M/nn/SpatialTransformer.cpp:136-139).
+int permute3D_0_2_1(hipStream_t stream, const DeviceBuffer &src, DeviceBuffer &dst, size_t isize,
+                    size_t jsize, size_t ksize);
+
 }  // namespace msd

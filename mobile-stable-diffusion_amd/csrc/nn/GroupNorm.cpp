@@ -60,6 +60,25 @@ int GroupNorm::forward(const DeviceBuffer &input, const DeviceBuffer &chunk, Dev
     return run(input, &chunk, output, num_events_in_list, event_wait_list, event);
 }
 
+int GroupNorm::forwardTokens(const DeviceBuffer &input, DeviceBuffer &output, unsigned num_events_in_list,
+                             const hipEvent_t *event_wait_list, hipEvent_t event) {
+    if (bufferWeight.empty() || bufferBias.empty()) throw std::runtime_error("GroupNorm: init() not called");
+    checkInput(input.bytes(), input.dtype());
+    if (output.bytes() != input.bytes() || output.dtype() != input.dtype() || output.ptr() == input.ptr())
+        throw std::runtime_error("output must be separate memory of the input's size / type");
+    for (unsigned i = 0; i < num_events_in_list; i++) {
+        const hipError_t err = hipStreamWaitEvent(stream, event_wait_list[i], 0);
+        if (err != hipSuccess) return (int)err;
+    }
+    const size_t channelSize = input.count() / batch / num_channels;
+    const int rc = msd_groupnorm_tokens(input.ptr(), output.ptr(), static_cast<const float *>(bufferWeight.ptr()),
+                                        static_cast<const float *>(bufferBias.ptr()), batch, num_channels,
+                                        channelSize, num_groups, eps, (int)input.dtype(), stream);
+    if (rc != MSD_OK) return rc;
+    if (event) return (int)hipEventRecord(event, stream);
+    return MSD_OK;
+}
+
 int GroupNorm::run(const DeviceBuffer &input, const DeviceBuffer *chunk, DeviceBuffer &output,
                    unsigned num_events_in_list, const hipEvent_t *event_wait_list, hipEvent_t event) {
     if (bufferWeight.empty() || bufferBias.empty()) throw std::runtime_error("GroupNorm: init() not called");

@@ -50,6 +50,13 @@ public:
                 unsigned num_events_in_list = 0, const hipEvent_t *event_wait_list = nullptr,
                 hipEvent_t event = nullptr);
 
+    // GroupNorm stored token-major: output[b, p, c] = GroupNorm(input)[b, c, p], i.e. forward()
+    // followed by the (0, 2, 1) permute of SpatialTransformer::forward
+    // (M/nn/SpatialTransformer.cpp:127-139) in one launch.  Never applies SiLU.  output must
+    // be different memory of the same size.
+    int forwardTokens(const DeviceBuffer &input, DeviceBuffer &output, unsigned num_events_in_list = 0,
+                      const hipEvent_t *event_wait_list = nullptr, hipEvent_t event = nullptr);
+
     // The precondition checks of forward() alone (no device work).
     void checkInput(size_t input_bytes, DType dtype) const;
 

@@ -99,6 +99,12 @@ int msdnn_groupnorm_forward_chunk(void *h, void *in, void *chunk, size_t chunk_b
         return static_cast<GroupNorm *>(h)->forward(i, c, o);
     });
 }
+int msdnn_groupnorm_forward_tokens(void *h, void *in, void *out, size_t bytes, int dtype) {
+    return guarded([&] {
+        DeviceBuffer i = wrap(in, bytes, dtype), o = wrap(out, bytes, dtype);
+        return static_cast<GroupNorm *>(h)->forwardTokens(i, o);
+    });
+}
 void msdnn_groupnorm_destroy(void *h) { delete static_cast<GroupNorm *>(h); }
 
 // ---- LayerNorm

@@ -144,6 +144,17 @@ def test_objects_with_fused_adds(msd, nn, orc, cuda, tmp_path):
     assert "chunk size" in msd.nn_last_error()
     nn.msdnn_groupnorm_destroy(g)
 
+    # SpatialTransformer's norm (eps 1e-6, no SiLU) written token-major (M/nn/SpatialTransformer.cpp:127-139)
+    g = nn.msdnn_groupnorm_create(None, 32, channels, 1e-6, b"out_w.npy", b"out_b.npy", batch, 0)
+    assert nn.msdnn_groupnorm_init(g) == 0, msd.nn_last_error()
+    xd = _dev(x, cuda, True)
+    td = torch.empty((batch, hw, channels), dtype=torch.float16, device=cuda)
+    assert nn.msdnn_groupnorm_forward_tokens(g, _ptr(xd), _ptr(td), nbytes, 1) == 0, msd.nn_last_error()
+    ref = orc.groupnorm(x, w, b, 32, 1e-6, silu=False)
+    assert_close_f16(td.float().cpu().numpy(), orc.round_to_half(ref).transpose(0, 2, 1))
+    assert nn.msdnn_groupnorm_forward_tokens(g, _ptr(xd), _ptr(xd), nbytes, 1) < 0  # needs separate output
+    nn.msdnn_groupnorm_destroy(g)
+
     dim, rows = 640, 2048
     lw = orc.normal((dim,), seed=45, mean=1.0, sigma=0.1)
     lb = orc.normal((dim,), seed=46, sigma=0.1)
