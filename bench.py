@@ -27,7 +27,7 @@ if REPO not in sys.path:
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # measured HBM bytes per geglu_kernel<__half> launch, averaged over the 16 launches of a step
 # (rocprofv3 counters; algorithmic figure is 34652160)
-GEGLU_TRAFFIC_BYTES_PER_LAUNCH = 34745208
+GEGLU_TRAFFIC_BYTES_PER_LAUNCH = 34683002
 
 
 # ----------------------------------------------------------------------------
@@ -505,7 +505,7 @@ def main():
     # launch was measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, calibrated on a plain
     # 64 MiB copy (FETCH_SIZE x 1.9992, WRITE_SIZE x 1.0000).
     dk = families["geglu"]
-    roofline = {"bound": "hbm", "kernel": "geglu_kernel<__half>", "achieved": dk["GBps"], "peak": HBM_PEAK_GBS,
+    roofline = {"bound": "hbm", "kernel": "geglu_kernel<__half, 1>", "achieved": dk["GBps"], "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(dk["GBps"] / HBM_PEAK_GBS, 4),
                 "bytes_per_launch": dk["bytes"] // dk["launches"], "us_per_launch": dk["us_per_launch"],
                 "traffic": GEGLU_TRAFFIC_BYTES_PER_LAUNCH}

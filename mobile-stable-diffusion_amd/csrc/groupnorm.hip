@@ -468,16 +468,6 @@ __global__ __launch_bounds__(kGenericThreads) void gn_tokens_generic_kernel(
 // ---------------------------------------------------------------------------
 // Host: launch plan
 // ---------------------------------------------------------------------------
-FastDiv make_fast_div(uint32_t d) {
-    FastDiv fd{0u, 0u, d};
-    if (d <= 1) return fd;
-    uint32_t L = 0;
-    while ((1ull << L) < d) L++;
-    fd.mul = (uint32_t)(((1ull << (31 + L)) + d - 1) / d);
-    fd.shift = L - 1;
-    return fd;
-}
-
 const int kKValues[] = {1, 2, 3, 4, 5, 6, 8, 10, 12, 16};
 
 inline int round_up_k(uint32_t k) {

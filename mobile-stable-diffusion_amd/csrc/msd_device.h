@@ -103,6 +103,17 @@ struct FastDiv {
     uint32_t d;
 };
 
+// Host side: the constants for divisor d.
+inline FastDiv make_fast_div(uint32_t d) {
+    FastDiv fd{0u, 0u, d};
+    if (d <= 1) return fd;
+    uint32_t L = 0;
+    while ((1ull << L) < d) L++;
+    fd.mul = (uint32_t)(((1ull << (31 + L)) + d - 1) / d);
+    fd.shift = L - 1;
+    return fd;
+}
+
 __device__ __forceinline__ uint32_t fast_div(uint32_t n, const FastDiv &fd) {
     const uint32_t q = __umulhi(n, fd.mul) >> fd.shift;
     return fd.mul == 0 ? n : q;

@@ -11,16 +11,6 @@
 namespace msd {
 namespace {
 
-FastDiv make_fast_div(uint32_t d) {
-    FastDiv fd{0u, 0u, d};
-    if (d <= 1) return fd;
-    uint32_t L = 0;
-    while ((1ull << L) < d) L++;
-    fd.mul = (uint32_t)(((1ull << (31 + L)) + d - 1) / d);
-    fd.shift = L - 1;
-    return fd;
-}
-
 constexpr int kStreamThreads = 256;
 constexpr int kStreamUnroll = 1;  // vectors per lane of the elementwise kernels
 
