@@ -184,6 +184,60 @@ int msd_timestep_embedding(const int64_t *timesteps, void *out, size_t batch, si
  */
 int msd_ddim_timesteps(int ddim_num_steps, int *out, int cap);
 
+/*
+ * Linear layer on the few rows of the time embedding: y[m, n] = act_out(act_in(x)[m, k] .
+ * weight[n, k]^T + bias[n]), m <= 8 (larger m is a GEMM and is rejected).  x, weight and y
+ * are in the storage type `dtype`, bias is float32 or NULL, accumulation is float32.
+ * Replaces Linear::forward (M/nn/Linear.cpp:74-289, kernel K/linear.cl:345-430) at its
+ * embedding call sites together with the silu enqueue next to it:
+ *   act_out = MSD_ACT_SILU : time_embed_0 then silu   (M/UNetModel.cpp:1107-1117)
+ *   no activation          : time_embed_2              (M/UNetModel.cpp:1119-1120)
+ *   act_in = MSD_ACT_SILU  : silu(emb) then embed_linear, per ResBlock
+ *                            (M/nn/ResBlock.cpp:173-183)
+ * The reference adds the k products in ascending order into one accumulator; here each of
+ * 64 lanes adds its share in ascending order and a fixed tree adds the lanes (agreement
+ * within float32 summation error, see the tests).  y must not overlap x
+ * (M/nn/Linear.cpp:78-81).
+ */
+#define MSD_ACT_NONE 0
+#define MSD_ACT_SILU 1
+int msd_linear_rows(const void *x, const void *weight, const float *bias, void *y, size_t m,
+                    size_t n, size_t k, int act_in, int act_out, int dtype, void *stream);
+
+/*
+ * Row softmax over the last dimension of [rows, cols]; y may alias x (every reference
+ * call site is in place).  Replaces the softmax kernel K/util.cl:150-187 enqueued by
+ * CrossAttention::forward (M/nn/CrossAttention.cpp:362-377) and AttnBlock::forward
+ * (M/nn/AttnBlock.cpp:196-206).  stable = 0 computes exp(x) / sum exp(x) as that kernel
+ * does (overflowing to inf / nan where it does, x > 88.7); stable != 0 subtracts the row
+ * maximum first, which is the same value wherever the former is finite.
+ */
+int msd_softmax(const void *x, void *y, size_t rows, size_t cols, int stable, int dtype,
+                void *stream);
+
+/*
+ * DDIM sampler arithmetic (M/DDIMSampler.cpp).  Host only:
+ *   msd_alphas_cumprod  the 1000 cumulative alpha products of the constructor (:18-39):
+ *                       betas = linspace(sqrt(0.00085), sqrt(0.0120), 1000)^2 and the
+ *                       running product of 1 - beta in double, stored as float.
+ *   msd_ddim_schedule   msd_ddim_timesteps plus make_schedule (:123-137) and :68-71:
+ *                       alphas[i] = cumprod[t_i], alphas_prev = {cumprod[0], cumprod[t_0],
+ *                       ...}, sqrt_one_minus_alphas[i] = sqrt(1 - alphas[i]).  Writes at most
+ *                       cap entries per array and returns the full count; -1 for steps
+ *                       outside [1, 1000]; -2 when the list would contain 1000 (steps > 500),
+ *                       where the reference indexes one past its table.
+ * On the stream:
+ *   msd_ddim_update     x_prev = sqrt(a_prev) * ((x - sqrt_one_minus_at * e_t) / sqrt(a_t))
+ *                       + sqrt(1 - a_prev) * e_t, the three loops of p_sample_ddim (:107-118,
+ *                       eta 0) in one pass, every operation rounded separately in that order
+ *                       (bit-identical to the host loops for float32).  x_prev may alias x.
+ */
+int msd_alphas_cumprod(float *out_1000);
+int msd_ddim_schedule(int ddim_num_steps, int *timesteps, float *alphas, float *alphas_prev,
+                      float *sqrt_one_minus_alphas, int cap);
+int msd_ddim_update(const void *x, const void *e_t, void *x_prev, size_t n, float a_t,
+                    float a_prev, float sqrt_one_minus_at, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -26,7 +26,9 @@ C_ABI_SYMBOLS = (
     "msd_silu", "msd_gelu", "msd_quick_gelu", "msd_timestep_embedding", "msd_ddim_timesteps",
     "msd_elemwise_add", "msd_chunkwise_add", "msd_chunk_add_groupnorm", "msd_add_layernorm", "msd_copy",
     "msd_groupnorm_tokens", "msd_permute_0_2_1",
+    "msd_linear_rows", "msd_softmax", "msd_alphas_cumprod", "msd_ddim_schedule", "msd_ddim_update",
 )
+ACT_NONE, ACT_SILU = 0, 1
 
 _lib = None
 
@@ -68,6 +70,12 @@ def load_library(path=None):
         getattr(lib, name).argtypes = [vp, vp, sz, it, vp]
     lib.msd_timestep_embedding.argtypes = [vp, vp, sz, sz, fl, it, vp]
     lib.msd_ddim_timesteps.argtypes = [it, ctypes.POINTER(ctypes.c_int), it]
+    lib.msd_linear_rows.argtypes = [vp, vp, vp, vp, sz, sz, sz, it, it, it, vp]
+    lib.msd_softmax.argtypes = [vp, vp, sz, sz, it, it, vp]
+    flp, inp = ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_int)
+    lib.msd_alphas_cumprod.argtypes = [flp]
+    lib.msd_ddim_schedule.argtypes = [it, inp, flp, flp, flp, it]
+    lib.msd_ddim_update.argtypes = [vp, vp, vp, sz, fl, fl, fl, it, vp]
     for name in C_ABI_SYMBOLS:
         if name != "msd_error_string":
             getattr(lib, name).restype = it
@@ -238,6 +246,58 @@ def ddim_timesteps(steps):
     buf = (ctypes.c_int * n)()
     lib.msd_ddim_timesteps(steps, buf, n)
     return list(buf)
+
+
+def linear_rows(x, weight, bias=None, act_in=ACT_NONE, act_out=ACT_NONE, out=None):
+    """x [m <= 8, k], weight [n, k] (x's dtype), bias float32 [n] or None -> [m, n]."""
+    import torch
+    m, k = x.shape
+    n = weight.shape[0]
+    if weight.shape[1] != k or weight.dtype != x.dtype:
+        raise MsdError("weight must be [n, k] in the dtype of x")
+    out = torch.empty((m, n), dtype=x.dtype, device=x.device) if out is None else out
+    bp = _dev(bias) if bias is not None else None
+    check(load_library().msd_linear_rows(_dev(x), _dev(weight), bp, _dev(out), m, n, k, act_in, act_out,
+                                         _dtype_code(x), _stream()))
+    return out
+
+
+def softmax(x, stable=False, out=None):
+    """Softmax over the last axis; out may be x (in place)."""
+    import torch
+    out = torch.empty_like(x) if out is None else out
+    cols = x.shape[-1]
+    rows = x.numel() // cols if cols else 0
+    check(load_library().msd_softmax(_dev(x), _dev(out), rows, cols, int(stable), _dtype_code(x), _stream()))
+    return out
+
+
+def alphas_cumprod():
+    """The sampler's 1000 cumulative alpha products as a list of floats (host only)."""
+    buf = (ctypes.c_float * 1000)()
+    check(load_library().msd_alphas_cumprod(buf))
+    return list(buf)
+
+
+def ddim_schedule(steps):
+    """-> (timesteps, alphas, alphas_prev, sqrt_one_minus_alphas) as lists (host only)."""
+    lib = load_library()
+    n = lib.msd_ddim_schedule(steps, None, None, None, None, 0)
+    if n < 0:
+        raise MsdError("ddim steps must be in [1, 500] (code %d)" % n)
+    ts = (ctypes.c_int * n)()
+    a, ap, s1m = (ctypes.c_float * n)(), (ctypes.c_float * n)(), (ctypes.c_float * n)()
+    lib.msd_ddim_schedule(steps, ts, a, ap, s1m, n)
+    return list(ts), list(a), list(ap), list(s1m)
+
+
+def ddim_update(x, e_t, a_t, a_prev, sqrt_one_minus_at, out=None):
+    """One DDIM step (eta 0) on device tensors; out may be x."""
+    import torch
+    out = torch.empty_like(x) if out is None else out
+    check(load_library().msd_ddim_update(_dev(x), _dev(e_t), _dev(out), x.numel(), a_t, a_prev,
+                                         sqrt_one_minus_at, _dtype_code(x), _stream()))
+    return out
 
 
 # ---------------------------------------------------------------------------------------

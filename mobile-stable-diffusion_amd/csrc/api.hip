@@ -297,4 +297,71 @@ int msd_ddim_timesteps(int ddim_num_steps, int *out, int cap) {
     return count;
 }
 
+int msd_linear_rows(const void *x, const void *weight, const float *bias, void *y, size_t m,
+                    size_t n, size_t k, int act_in, int act_out, int dtype, void *stream) {
+    if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
+    if ((act_in != MSD_ACT_NONE && act_in != MSD_ACT_SILU) ||
+        (act_out != MSD_ACT_NONE && act_out != MSD_ACT_SILU))
+        return MSD_ERR_INVALID_VALUE;
+    if (m > 8) return MSD_ERR_INVALID_VALUE;
+    if (m * n != 0 && (!y || (k != 0 && (!x || !weight)) || x == y)) return MSD_ERR_INVALID_VALUE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == MSD_DTYPE_F32)
+        return linear_rows_dispatch<float>(x, weight, bias, y, m, n, k, act_in, act_out, s);
+    return linear_rows_dispatch<__half>(x, weight, bias, y, m, n, k, act_in, act_out, s);
+}
+
+int msd_softmax(const void *x, void *y, size_t rows, size_t cols, int stable, int dtype,
+                void *stream) {
+    if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
+    if (rows * cols != 0 && (!x || !y)) return MSD_ERR_INVALID_VALUE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == MSD_DTYPE_F32) return softmax_dispatch<float>(x, y, rows, cols, stable != 0, s);
+    return softmax_dispatch<__half>(x, y, rows, cols, stable != 0, s);
+}
+
+int msd_alphas_cumprod(float *out_1000) {
+    if (!out_1000) return MSD_ERR_INVALID_VALUE;
+    const int steps = 1000;
+    const double linear_start = 0.00085, linear_end = 0.0120;
+    const double first = std::sqrt(linear_start), last = std::sqrt(linear_end);
+    const double spacing = (last - first) / static_cast<double>(steps - 1);
+    double product = 1.0;
+    for (int i = 0; i < steps; i++) {
+        const double root = first + static_cast<double>(i) * spacing;
+        product *= 1.0 - root * root;
+        out_1000[i] = static_cast<float>(product);
+    }
+    return MSD_OK;
+}
+
+int msd_ddim_schedule(int ddim_num_steps, int *timesteps, float *alphas, float *alphas_prev,
+                      float *sqrt_one_minus_alphas, int cap) {
+    static float cumprod[1000];
+    static std::once_flag once;
+    std::call_once(once, [] { (void)msd_alphas_cumprod(cumprod); });
+    int local[1001];
+    const int count = msd_ddim_timesteps(ddim_num_steps, local, 1001);
+    if (count < 0) return -1;
+    if (local[count - 1] >= 1000) return -2;
+    for (int i = 0; i < count && i < cap; i++) {
+        const float a = cumprod[local[i]];
+        if (timesteps) timesteps[i] = local[i];
+        if (alphas) alphas[i] = a;
+        if (alphas_prev) alphas_prev[i] = i == 0 ? cumprod[0] : cumprod[local[i - 1]];
+        if (sqrt_one_minus_alphas) sqrt_one_minus_alphas[i] = std::sqrt(1.0f - a);
+    }
+    return count;
+}
+
+int msd_ddim_update(const void *x, const void *e_t, void *x_prev, size_t n, float a_t,
+                    float a_prev, float sqrt_one_minus_at, int dtype, void *stream) {
+    if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
+    if (n != 0 && (!x || !e_t || !x_prev)) return MSD_ERR_INVALID_VALUE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == MSD_DTYPE_F32)
+        return ddim_update_dispatch<float>(x, e_t, x_prev, n, a_t, a_prev, sqrt_one_minus_at, s);
+    return ddim_update_dispatch<__half>(x, e_t, x_prev, n, a_t, a_prev, sqrt_one_minus_at, s);
+}
+
 }  // extern "C"

@@ -154,6 +154,23 @@ __device__ __forceinline__ float team_sum(float v) {
 
 __device__ __forceinline__ float wave_sum(float v) { return team_sum<64>(v); }
 
+// Maximum over aligned teams of TL lanes, same exchange pattern as team_sum.
+template <int TL>
+__device__ __forceinline__ float team_max(float v) {
+    static_assert(TL == 4 || TL == 8 || TL == 16 || TL == 32 || TL == 64, "team size");
+    v = fmaxf(v, dpp_move<kDppXor1>(v));
+    v = fmaxf(v, dpp_move<kDppXor2>(v));
+    if (TL >= 8) v = fmaxf(v, dpp_move<kDppHalfMirror>(v));
+    if (TL >= 16) v = fmaxf(v, dpp_move<kDppRowMirror>(v));
+    if (TL >= 32) v = fmaxf(v, __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401F)));
+    if (TL >= 64) {
+        const float lo = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+        const float hi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+        v = fmaxf(lo, hi);
+    }
+    return v;
+}
+
 // Sum over a workgroup of NW wavefronts; `slots` is NW floats of LDS that no
 // other reduction in flight uses.  One barrier; every thread gets the total.
 template <int NW>

@@ -68,4 +68,14 @@ template <typename T>
 int temb_dispatch(const int64_t *timesteps, void *out, size_t batch, size_t dim, float max_period,
                   hipStream_t stream);
 
+// y[m, n] = act_out(act_in(x) . w^T + bias), m <= 8; activations: 0 none, 1 SiLU
+template <typename T>
+int linear_rows_dispatch(const void *x, const void *w, const float *bias, void *y, size_t m, size_t n,
+                         size_t k, int act_in, int act_out, hipStream_t stream);
+template <typename T>
+int softmax_dispatch(const void *x, void *y, size_t rows, size_t cols, int stable, hipStream_t stream);
+template <typename T>
+int ddim_update_dispatch(const void *x, const void *e_t, void *x_prev, size_t n, float a_t,
+                         float a_prev, float sqrt_one_minus_at, hipStream_t stream);
+
 }  // namespace msd

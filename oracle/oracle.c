@@ -12,6 +12,7 @@
 #include "oracle.h"
 
 #include <math.h>
+#include <stdlib.h>
 #include <string.h>
 #ifdef _OPENMP
 #include <omp.h>
@@ -416,6 +417,139 @@ void orc64_timestep_embedding(int64_t timestep, double *out, int dim, double max
         const double freq = exp(-log(max_period) * (double)i / (double)half);
         out[i] = cos((double)timestep * freq);
         out[i + half] = sin((double)timestep * freq);
+    }
+}
+
+/* ------------------------------------------------------------------ */
+/* neighbours of the path: embedding Linear, row softmax, DDIM schedule */
+/* ------------------------------------------------------------------ */
+
+/* K/linear.cl:345-430 (tile_reg_n_vector_linear, the variant LINEAR_KERNEL_VERSION 4
+ * of M/setting.h:8 selects, M/nn/Linear.cpp:244-289): C[i,j] = sum_k A[i,k]*B[j,k],
+ * one float accumulator per output, k ascending, bias added last. */
+void orc_linear(const float *a, const float *w, const float *bias, float *c, size_t m, size_t n,
+                size_t k) {
+#pragma omp parallel for collapse(2) schedule(static)
+    for (size_t i = 0; i < m; i++)
+        for (size_t j = 0; j < n; j++) {
+            float acc = 0.0f;
+            for (size_t kk = 0; kk < k; kk++) acc += a[i * k + kk] * w[j * k + kk];
+            if (bias != NULL) acc += bias[j];
+            c[i * n + j] = acc;
+        }
+}
+
+void orc64_linear(const float *a, const float *w, const float *bias, double *c, size_t m, size_t n,
+                  size_t k) {
+    for (size_t i = 0; i < m; i++)
+        for (size_t j = 0; j < n; j++) {
+            double acc = 0.0;
+            for (size_t kk = 0; kk < k; kk++) acc += (double)a[i * k + kk] * (double)w[j * k + kk];
+            if (bias != NULL) acc += (double)bias[j];
+            c[i * n + j] = acc;
+        }
+}
+
+/* K/util.cl:150-187: one workgroup of local_size lanes per chunk; lane-strided
+ * partial sums of exp(x) (no maximum is subtracted), the tree of :172-180 with its
+ * odd-size bookkeeping, then exp(x) / total.  The call sites use 64 lanes
+ * (M/nn/CrossAttention.cpp:362-377, M/nn/AttnBlock.cpp:196-206). */
+void orc_softmax(const float *input, float *output, size_t rows, size_t chunk_size,
+                 size_t local_size) {
+#pragma omp parallel for schedule(static)
+    for (size_t wg = 0; wg < rows; wg++) {
+        const float *in = input + wg * chunk_size;
+        float *out = output + wg * chunk_size;
+        float sums[1024];
+        float cache_small[4096];
+        float *cache = chunk_size <= 4096 ? cache_small : (float *)malloc(chunk_size * sizeof(float));
+        for (size_t lid = 0; lid < local_size; lid++) {
+            float sum = 0.0f;
+            for (size_t index = lid; index < chunk_size; index += local_size) {
+                const float e = expf(in[index]);
+                sum += e;
+                cache[index] = e;
+            }
+            sums[lid] = sum;
+        }
+        size_t remainder = local_size % 2;
+        for (size_t offset = local_size / 2; offset > 0; offset /= 2) {
+            for (size_t lid = 0; lid < offset; lid++)
+                sums[lid + remainder] += sums[lid + offset + remainder];
+            offset += remainder;
+            remainder = offset % 2;
+        }
+        for (size_t index = 0; index < chunk_size; index++) out[index] = cache[index] / sums[0];
+        if (cache != cache_small) free(cache);
+    }
+}
+
+/* textbook softmax with the row maximum subtracted, float64 */
+void orc64_softmax(const float *input, double *output, size_t rows, size_t chunk_size) {
+    for (size_t r = 0; r < rows; r++) {
+        const float *in = input + r * chunk_size;
+        double mx = -INFINITY, total = 0.0;
+        for (size_t i = 0; i < chunk_size; i++) mx = in[i] > mx ? in[i] : mx;
+        for (size_t i = 0; i < chunk_size; i++) total += exp((double)in[i] - mx);
+        for (size_t i = 0; i < chunk_size; i++)
+            output[r * chunk_size + i] = exp((double)in[i] - mx) / total;
+    }
+}
+
+/* M/DDIMSampler.cpp:18-39: betas = linspace(sqrt(0.00085), sqrt(0.0120), 1000)^2 in
+ * double (linspace at :139-153), alphas = 1 - beta, running product in double,
+ * stored as float. */
+void orc_alphas_cumprod(float *out) {
+    const int steps = 1000;
+    const double start = sqrt(0.00085), end = sqrt(0.0120);
+    const double step_size = (end - start) / (double)(steps - 1);
+    double acc = 1.0;
+    for (int i = 0; i < steps; i++) {
+        double beta = start + (double)i * step_size;
+        beta = beta * beta;
+        const double alpha = 1.0f - beta;
+        acc = i == 0 ? alpha : acc * alpha;
+        out[i] = (float)acc;
+    }
+}
+
+/* M/DDIMSampler.cpp:60-76 with make_schedule (:123-137): alphas[i] = cumprod[ts[i]],
+ * alphas_prev = {cumprod[0], cumprod[ts[0]], ...}, sqrt(1 - alphas).  Returns the
+ * count, -1 for steps outside [1, 1000], -2 when the list reaches 1000 (the
+ * reference would index one past its 1000-entry table). */
+int orc_ddim_schedule(int ddim_num_steps, int *timesteps, float *alphas, float *alphas_prev,
+                      float *sqrt_one_minus_alphas, int cap) {
+    int ts[1001];
+    const int count = orc_ddim_timesteps(ddim_num_steps, ts, 1001);
+    if (count < 0) return -1;
+    if (ts[count - 1] >= 1000) return -2;
+    float cumprod[1000];
+    orc_alphas_cumprod(cumprod);
+    for (int i = 0; i < count && i < cap; i++) {
+        timesteps[i] = ts[i];
+        alphas[i] = cumprod[ts[i]];
+        alphas_prev[i] = i == 0 ? cumprod[0] : cumprod[ts[i - 1]];
+        sqrt_one_minus_alphas[i] = sqrtf(1.0f - alphas[i]);
+    }
+    return count;
+}
+
+/* M/DDIMSampler.cpp:94-121 (eta = 0): three float loops; sqrt on float values
+ * (the reference builds with libc++, whose ::sqrt(float) is the float overload). */
+void orc_ddim_update(const float *x, const float *e_t, float *x_prev, size_t n, float a_t,
+                     float a_prev, float sqrt_one_minus_at) {
+    for (size_t i = 0; i < n; i++) {
+        const float pred_x0 = (x[i] - sqrt_one_minus_at * e_t[i]) / sqrtf(a_t);
+        const float dir_xt = sqrtf(1.0f - a_prev) * e_t[i];
+        x_prev[i] = sqrtf(a_prev) * pred_x0 + dir_xt;
+    }
+}
+
+void orc64_ddim_update(const float *x, const float *e_t, double *x_prev, size_t n, double a_t,
+                       double a_prev) {
+    for (size_t i = 0; i < n; i++) {
+        const double pred_x0 = ((double)x[i] - sqrt(1.0 - a_t) * (double)e_t[i]) / sqrt(a_t);
+        x_prev[i] = sqrt(a_prev) * pred_x0 + sqrt(1.0 - a_prev) * (double)e_t[i];
     }
 }
 

@@ -24,6 +24,14 @@
  *        literal 981 (native-lib.cpp:240) as the first step of 50.
  *   orc_elemwise_add, orc_chunkwise_add, orc_permute3D_0_2_1 : exact; checked against numpy
  *        broadcasting / transpose (bit-exact).
+ *   orc_linear : torch.nn.functional.linear fixtures (non-square, with and without
+ *        bias), orc64 brute force, one-hot rows that select single weights.
+ *   orc_softmax : torch.softmax fixtures, rows sum to 1, shift invariance against the
+ *        max-subtracting float64 textbook form, odd workgroup sizes against a plain sum.
+ *   orc_alphas_cumprod, orc_ddim_schedule : the LDM "linear" beta schedule computed by
+ *        torch in float64 (fixture), first / last known values, alphas_prev shift.
+ *   orc_ddim_update : float64 fixture of the LDM DDIM step (eta 0), e_t = 0 and
+ *        a_prev = a_t special cases.
  *   orc_quick_gelu : PARITY UNPINNED BY THE REFERENCE (the reference has no
  *        quick_GELU); pinned only by the closed form x*sigmoid(1.702x).
  */
@@ -108,6 +116,27 @@ void orc64_gelu(const float *x, double *y, size_t n);
 void orc64_quick_gelu(const float *x, double *y, size_t n);
 void orc64_geglu(const float *ab, double *y, size_t rows, size_t inner);
 void orc64_timestep_embedding(int64_t timestep, double *out, int dim, double max_period);
+
+/* ---- neighbours of the path (the callers either side of it) ---- */
+/* K/linear.cl:345-430 via M/nn/Linear.cpp:244-289: c[m,n] = a[m,k] . w[n,k]^T + bias; bias may be NULL */
+void orc_linear(const float *a, const float *w, const float *bias, float *c, size_t m, size_t n,
+                size_t k);
+void orc64_linear(const float *a, const float *w, const float *bias, double *c, size_t m, size_t n,
+                  size_t k);
+/* K/util.cl:150-187 with a workgroup of local_size (<= 1024) lanes per chunk */
+void orc_softmax(const float *input, float *output, size_t rows, size_t chunk_size,
+                 size_t local_size);
+void orc64_softmax(const float *input, double *output, size_t rows, size_t chunk_size);
+/* M/DDIMSampler.cpp:18-39: out[1000] */
+void orc_alphas_cumprod(float *out);
+/* M/DDIMSampler.cpp:60-76,123-137; returns the count (-1 bad steps, -2 table overrun) */
+int orc_ddim_schedule(int ddim_num_steps, int *timesteps, float *alphas, float *alphas_prev,
+                      float *sqrt_one_minus_alphas, int cap);
+/* M/DDIMSampler.cpp:94-121 */
+void orc_ddim_update(const float *x, const float *e_t, float *x_prev, size_t n, float a_t,
+                     float a_prev, float sqrt_one_minus_at);
+void orc64_ddim_update(const float *x, const float *e_t, double *x_prev, size_t n, double a_t,
+                       double a_prev);
 
 /* ---- threading control for the CPU-baseline leg ---- */
 int orc_max_threads(void);

@@ -69,6 +69,14 @@ def lib():
         "orc64_quick_gelu": (None, [_f32p, _f64p, _sz]),
         "orc64_geglu": (None, [_f32p, _f64p, _sz, _sz]),
         "orc64_timestep_embedding": (None, [_i64, _f64p, _it, _db]),
+        "orc_linear": (None, [_f32p, _f32p, ctypes.c_void_p, _f32p, _sz, _sz, _sz]),
+        "orc64_linear": (None, [_f32p, _f32p, ctypes.c_void_p, _f64p, _sz, _sz, _sz]),
+        "orc_softmax": (None, [_f32p, _f32p, _sz, _sz, _sz]),
+        "orc64_softmax": (None, [_f32p, _f64p, _sz, _sz]),
+        "orc_alphas_cumprod": (None, [_f32p]),
+        "orc_ddim_schedule": (_it, [_it, _i32p, _f32p, _f32p, _f32p, _it]),
+        "orc_ddim_update": (None, [_f32p, _f32p, _f32p, _sz, _fl, _fl, _fl]),
+        "orc64_ddim_update": (None, [_f32p, _f32p, _f64p, _sz, _db, _db]),
         "orc_max_threads": (_it, []),
         "orc_set_threads": (None, [_it]),
     }
@@ -219,6 +227,90 @@ def ddim_timesteps(steps):
     if n < 0:
         raise ValueError("steps out of range")
     return buf[:n].tolist()
+
+
+# ---------------------------------------------------------------- neighbours of the path
+def _bias_ptr(bias):
+    if bias is None:
+        return None, None
+    b = np.ascontiguousarray(bias, dtype=np.float32).reshape(-1)
+    return b, b.ctypes.data_as(ctypes.c_void_p)
+
+
+def linear(x, weight, bias=None):
+    """x [m, k], weight [n, k] -> [m, n] (float32, k ascending)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = np.ascontiguousarray(weight, dtype=np.float32)
+    m, k = x.shape
+    n = w.shape[0]
+    assert w.shape[1] == k
+    y = np.empty((m, n), dtype=np.float32)
+    keep, bp = _bias_ptr(bias)
+    lib().orc_linear(x.reshape(-1), w.reshape(-1), bp, y.reshape(-1), m, n, k)
+    return y
+
+
+def linear64(x, weight, bias=None):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = np.ascontiguousarray(weight, dtype=np.float32)
+    m, k = x.shape
+    n = w.shape[0]
+    y = np.empty((m, n), dtype=np.float64)
+    keep, bp = _bias_ptr(bias)
+    lib().orc64_linear(x.reshape(-1), w.reshape(-1), bp, y.reshape(-1), m, n, k)
+    return y
+
+
+def softmax(x, local_size=64):
+    """Row softmax over the last axis as the reference computes it (no max subtraction)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    chunk = x.shape[-1]
+    y = np.empty_like(x)
+    lib().orc_softmax(x.reshape(-1), y.reshape(-1), x.size // chunk, chunk, local_size)
+    return y
+
+
+def softmax64(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    chunk = x.shape[-1]
+    y = np.empty(x.shape, dtype=np.float64)
+    lib().orc64_softmax(x.reshape(-1), y.reshape(-1), x.size // chunk, chunk)
+    return y
+
+
+def alphas_cumprod():
+    out = np.empty(1000, dtype=np.float32)
+    lib().orc_alphas_cumprod(out)
+    return out
+
+
+def ddim_schedule(steps):
+    """-> (timesteps, alphas, alphas_prev, sqrt_one_minus_alphas); ValueError as the C code says."""
+    ts = np.zeros(1001, dtype=np.int32)
+    a = np.zeros(1001, dtype=np.float32)
+    ap = np.zeros(1001, dtype=np.float32)
+    s1m = np.zeros(1001, dtype=np.float32)
+    n = lib().orc_ddim_schedule(steps, ts, a, ap, s1m, 1001)
+    if n < 0:
+        raise ValueError("steps out of range" if n == -1 else "timestep list reaches 1000")
+    return ts[:n].copy(), a[:n].copy(), ap[:n].copy(), s1m[:n].copy()
+
+
+def ddim_update(x, e_t, a_t, a_prev, sqrt_one_minus_at):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    e = np.ascontiguousarray(e_t, dtype=np.float32)
+    y = np.empty_like(x)
+    lib().orc_ddim_update(x.reshape(-1), e.reshape(-1), y.reshape(-1), x.size, a_t, a_prev,
+                          sqrt_one_minus_at)
+    return y
+
+
+def ddim_update64(x, e_t, a_t, a_prev):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    e = np.ascontiguousarray(e_t, dtype=np.float32)
+    y = np.empty(x.shape, dtype=np.float64)
+    lib().orc64_ddim_update(x.reshape(-1), e.reshape(-1), y.reshape(-1), x.size, a_t, a_prev)
+    return y
 
 
 # ---------------------------------------------------------------- float64 textbook

@@ -2,8 +2,9 @@
 
 The reference ships no golden files (its .npy fixtures are git-ignored), so these
 vectors come from independent textbook implementations run once on the CPU:
-torch.nn.functional.{group_norm, layer_norm, silu, gelu} in float32 and the
-standard sinusoidal timestep-embedding formula in float64.  They pin the CPU
+torch.nn.functional.{group_norm, layer_norm, silu, gelu, linear}, torch.softmax in
+float32, the standard sinusoidal timestep-embedding formula and the LDM beta
+schedule / DDIM step in float64.  They pin the CPU
 oracle (tests/test_oracle_pinning.py) and are re-checked against the HIP
 kernels (tests/test_gpu_parity.py).  Inputs come from numpy's PCG64 with fixed
 seeds, so re-running this script reproduces the file bit for bit on the same
@@ -76,6 +77,41 @@ def main():
     args = ts[:, None].astype(np.float64) * freqs[None, :]
     fx["temb_t"] = ts
     fx["temb_f64"] = np.concatenate([np.cos(args), np.sin(args)], axis=1)
+
+    # ---- neighbours of the path (drawn after everything above, so the earlier arrays keep
+    # their values): Linear, row softmax, the LDM "linear" beta schedule and one DDIM step
+    for name, m, n, k, with_bias in [("lin_a", 2, 48, 320, True), ("lin_b", 2, 40, 1280, True),
+                                     ("lin_c", 3, 17, 96, False)]:
+        x = rng.standard_normal((m, k)).astype(np.float32)
+        w = (rng.standard_normal((n, k)) / np.sqrt(k)).astype(np.float32)
+        b = (0.1 * rng.standard_normal(n)).astype(np.float32) if with_bias else None
+        tb = torch.from_numpy(b) if with_bias else None
+        fx[name + "_x"], fx[name + "_w"] = x, w
+        if with_bias:
+            fx[name + "_b"] = b
+        fx[name + "_y"] = F.linear(torch.from_numpy(x), torch.from_numpy(w), tb).numpy()
+        fx[name + "_y_silu_in"] = F.linear(F.silu(torch.from_numpy(x)), torch.from_numpy(w), tb).numpy()
+        fx[name + "_y_silu_out"] = F.silu(F.linear(torch.from_numpy(x), torch.from_numpy(w), tb)).numpy()
+
+    for name, rows, cols, sigma in [("sm_a", 6, 77, 2.0), ("sm_b", 4, 256, 3.0), ("sm_c", 3, 1000, 1.0)]:
+        x = (rng.standard_normal((rows, cols)) * sigma).astype(np.float32)
+        fx[name + "_x"] = x
+        fx[name + "_y"] = torch.softmax(torch.from_numpy(x), dim=-1).numpy()
+
+    # LDM make_beta_schedule("linear", 1000, 0.00085, 0.0120) and its running product, float64
+    betas = torch.linspace(0.00085 ** 0.5, 0.0120 ** 0.5, 1000, dtype=torch.float64) ** 2
+    acp = torch.cumprod(1.0 - betas, dim=0)
+    fx["ddim_alphas_cumprod_f64"] = acp.numpy()
+    # one DDIM step (eta 0) of LDM's p_sample_ddim in float64 at step index 30 of 50
+    ddim_ts = np.arange(0, 1000, 1000 // 50) + 1
+    a_t, a_prev = float(acp[ddim_ts[30]]), float(acp[ddim_ts[29]])
+    x = rng.standard_normal(4 * 16 * 16).astype(np.float32)
+    e = rng.standard_normal(4 * 16 * 16).astype(np.float32)
+    xd, ed = torch.from_numpy(x).double(), torch.from_numpy(e).double()
+    pred_x0 = (xd - (1.0 - a_t) ** 0.5 * ed) / a_t ** 0.5
+    fx["ddim_x"], fx["ddim_e"] = x, e
+    fx["ddim_a_t"], fx["ddim_a_prev"] = np.float64(a_t), np.float64(a_prev)
+    fx["ddim_x_prev_f64"] = (a_prev ** 0.5 * pred_x0 + (1.0 - a_prev) ** 0.5 * ed).numpy()
 
     np.savez_compressed(OUT, **fx)
     print("wrote", OUT, os.path.getsize(OUT), "bytes,", len(fx), "arrays")
