@@ -368,6 +368,102 @@ def fusion_table(torch, msd, dev, stream):
     return rows
 
 
+def neighbour_table(torch, msd, dev, stream):
+    """The kernels either side of the path: attention row softmax (fp16, in place) next to a
+    plain copy of the same bytes, the Linear layers on the time-embedding rows with the SiLU
+    folded in or launched separately, and the DDIM latent update (graph-replayed)."""
+    import ctypes
+    vp = ctypes.c_void_p
+    lib = msd.load_library()
+    F16, F32 = msd.DTYPE_F16, msd.DTYPE_F32
+    rows = []
+
+    def sp():
+        return vp(torch.cuda.current_stream().cuda_stream)
+
+    def measure(fn, launches, budget=1500):
+        replay = capture(torch, msd, stream, fn)
+        with torch.cuda.stream(stream):
+            replay()
+            reps = max(2, int(budget // launches))
+            return event_time_ms(torch, replay, reps) * 1e3 / (reps * launches)
+
+    # softmax over keys: self-attention of the three UNet levels (batch 2 x 8 heads) and the
+    # cross-attention against 77 text tokens
+    for r, c in [(2 * 8 * 4096, 4096), (2 * 8 * 1024, 1024), (2 * 8 * 256, 256), (2 * 8 * 4096, 77),
+                 (2 * 8 * 1024, 77)]:
+        nbytes = 2 * r * c * 2
+        copies = max(2, min(64, int(1.2e9 // nbytes) + 1))
+        xs = [(torch.randn(r * c, device=dev) * 2.0).half() for _ in range(copies)]
+        ys = [torch.empty(r * c, device=dev, dtype=torch.float16) for _ in range(2)]
+
+        def body():
+            for x in xs:
+                assert lib.msd_softmax(vp(x.data_ptr()), vp(x.data_ptr()), r, c, 0, F16, sp()) == 0
+
+        def copy_body():
+            for i, x in enumerate(xs):
+                assert lib.msd_copy(vp(x.data_ptr()), vp(ys[i % 2].data_ptr()), r * c * 2, sp()) == 0
+        us, cus = measure(body, copies, 400), measure(copy_body, copies, 400)
+        gbs = nbytes / us / 1e3
+        rows.append({"kernel": "softmax", "shape": {"rows": r, "cols": c}, "dtype": "f16", "bytes": nbytes,
+                     "us": round(us, 2), "GBps": round(gbs, 1), "pct_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 1),
+                     "copy_us": round(cus, 2), "pct_of_copy_rate": round(100 * cus / us, 1)})
+        del xs, ys
+        torch.cuda.empty_cache()
+
+    # Linear on the two embedding rows; 16 weight sets in rotation (never cache-resident together
+    # with their predecessors at 1280 x 1280 fp32 = 6.5 MB each)
+    for n, k, what in [(1280, 320, "time_embed_0 + SiLU"), (1280, 1280, "time_embed_2"),
+                       (1280, 1280, "SiLU(emb) + embed_linear"), (320, 1280, "SiLU(emb) + embed_linear")]:
+        for dt, code, elt in ((torch.float16, F16, 2), (torch.float32, F32, 4)):
+            copies = 16
+            ws = [(torch.randn(n, k, device=dev) * k ** -0.5).to(dt) for _ in range(copies)]
+            bias = torch.zeros(n, device=dev)
+            x = torch.randn(BATCH, k, device=dev).to(dt)
+            tmp = torch.empty_like(x)
+            y = torch.empty(BATCH, n, device=dev, dtype=dt)
+            act_in = 1 if what.startswith("SiLU") else 0
+            act_out = 1 if what.endswith("SiLU") else 0
+
+            def fused():
+                for w in ws:
+                    assert lib.msd_linear_rows(vp(x.data_ptr()), vp(w.data_ptr()), vp(bias.data_ptr()),
+                                               vp(y.data_ptr()), BATCH, n, k, act_in, act_out, code, sp()) == 0
+
+            def separate():
+                for w in ws:
+                    src = x
+                    if act_in:
+                        assert lib.msd_silu(vp(x.data_ptr()), vp(tmp.data_ptr()), BATCH * k, code, sp()) == 0
+                        src = tmp
+                    assert lib.msd_linear_rows(vp(src.data_ptr()), vp(w.data_ptr()), vp(bias.data_ptr()),
+                                               vp(y.data_ptr()), BATCH, n, k, 0, 0, code, sp()) == 0
+                    if act_out:
+                        assert lib.msd_silu(vp(y.data_ptr()), vp(y.data_ptr()), BATCH * n, code, sp()) == 0
+            us = measure(fused, copies)
+            row = {"kernel": "linear_rows", "what": what, "shape": {"m": BATCH, "n": n, "k": k},
+                   "dtype": "f16" if elt == 2 else "f32", "bytes": n * k * elt, "us": round(us, 2),
+                   "GBps": round(n * k * elt / us / 1e3, 1)}
+            if act_in or act_out:
+                row["us_separate_silu"] = round(measure(separate, copies), 2)
+            rows.append(row)
+            del ws
+
+    # DDIM update of the latent, batch 2 x [4, 64, 64] float32, in place
+    n = BATCH * 4 * 64 * 64
+    x, e = torch.randn(n, device=dev), torch.randn(n, device=dev)
+
+    def ddim_body():
+        for _ in range(16):
+            assert lib.msd_ddim_update(vp(x.data_ptr()), vp(e.data_ptr()), vp(x.data_ptr()), n, 0.5, 0.6,
+                                       0.70710678, F32, sp()) == 0
+    rows.append({"kernel": "ddim_update", "shape": {"n": n}, "dtype": "f32", "bytes": 3 * n * 4,
+                 "us": round(measure(ddim_body, 16), 2)})
+    torch.cuda.empty_cache()
+    return rows
+
+
 def cpu_baseline(total_bytes, budget_s=12.0):
     """The reference path as host loops (the CPU oracle, fp32, unfused passes exactly as the
     reference enqueues them) over the layers of one full step, timed on this host's cores.
@@ -525,6 +621,7 @@ def main():
     if not args.no_shapes:
         out["shapes"] = shape_table(torch, msd, dev, stream)
         out["fusions"] = fusion_table(torch, msd, dev, stream)
+        out["neighbours"] = neighbour_table(torch, msd, dev, stream)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(step.bytes)
     else:

@@ -65,6 +65,7 @@ int msd_status(void *stream);
 #define MSD_TUNE_LN_THREADS 3    /* LayerNorm workgroup size: 64, 128, 256 or 512 */
 #define MSD_TUNE_GEGLU_VECTORS 4 /* 16-byte vectors per GEGLU lane: 1, 2 or 4 */
 #define MSD_TUNE_ACT_VECTORS 5   /* 16-byte vectors per lane of SiLU / GELU / quick_GELU: 1, 2 or 4 */
+#define MSD_TUNE_SOFTMAX_ROWS 6   /* rows per workgroup of the short-row softmax: 16, 32 or 64 */
 int msd_set_tuning(int knob, int value);
 
 /*

@@ -17,7 +17,8 @@ LIB_NN_PATH = os.path.join(CSRC_DIR, "libmsd_nn.so")
 
 DTYPE_F32 = 0
 DTYPE_F16 = 1
-TUNE_GN_SPLIT, TUNE_GN_THREADS, TUNE_LN_CHUNK, TUNE_LN_THREADS, TUNE_GEGLU_VECTORS, TUNE_ACT_VECTORS = range(6)
+TUNE_GN_SPLIT, TUNE_GN_THREADS, TUNE_LN_CHUNK, TUNE_LN_THREADS, TUNE_GEGLU_VECTORS, TUNE_ACT_VECTORS, \
+    TUNE_SOFTMAX_ROWS = range(7)
 
 # every symbol include/msd_hip.h declares
 C_ABI_SYMBOLS = (
@@ -304,6 +305,9 @@ def ddim_update(x, e_t, a_t, a_prev, sqrt_one_minus_at, out=None):
 # C++ layer objects (libmsd_nn.so) through their plain-C handles
 # ---------------------------------------------------------------------------------------
 _nn = None
+# int model(void *x, int t, void *e_t, size_t bytes, void *user): the sampler's noise-model callback
+MODEL_FN = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t,
+                            ctypes.c_void_p)
 
 
 def load_nn_library(path=None):
@@ -346,6 +350,14 @@ def load_nn_library(path=None):
         "msdnn_activation": (it, [vp, it, vp, vp, sz, it]),
         "msdnn_timestep_embedding": (it, [vp, lgp, sz, flp]),
         "msdnn_ddim_timesteps": (it, [it, ctypes.POINTER(ctypes.c_int), it]),
+        "msdnn_linear_create": (vp, [vp, sz, sz, cp, cp, it]),
+        "msdnn_linear_init": (it, [vp]),
+        "msdnn_linear_init_from": (it, [vp, flp, sz, flp, sz]),
+        "msdnn_linear_forward": (it, [vp, vp, sz, vp, sz, it, it, it]),
+        "msdnn_linear_destroy": (None, [vp]),
+        "msdnn_softmax": (it, [vp, vp, vp, sz, it, sz, it]),
+        "msdnn_ddim_sample": (it, [vp, vp, sz, it, it, MODEL_FN, vp, vp]),
+        "msdnn_ddim_make_schedule": (it, [ctypes.POINTER(ctypes.c_int), it, flp, flp]),
         "msdnn_test_buffer": (it, [vp, vp, sz, it, cp, flp, szp]),
         "msdnn_step_create": (vp, [vp, sz, it]),
         "msdnn_step_bytes": (sz, [vp]),

@@ -2,6 +2,7 @@
 
     libmsd_hip.so   HIP kernels + the C ABI declared in include/msd_hip.h
     libmsd_nn.so    C++ host layer objects (GroupNorm / LayerNorm / GEGLU / ...) on top of it
+    cli/msd_compare golden-file comparison tool (host only)
 
 Run as a script (`python build.py`) or call build_all().
 """
@@ -25,6 +26,7 @@ DEVICE_FLAGS = [
 
 LIB_HIP = os.path.join(CSRC, "libmsd_hip.so")
 LIB_NN = os.path.join(CSRC, "libmsd_nn.so")
+CLI_COMPARE = os.path.join(CSRC, "cli", "msd_compare")
 
 
 def _run(cmd):
@@ -70,11 +72,20 @@ def build_nn():
     return LIB_NN
 
 
+def build_cli():
+    """msd_compare: host-only golden-file comparison tool (no HIP, no GPU)."""
+    nn_dir = os.path.join(CSRC, "nn")
+    _run([os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-Wall", "-I", nn_dir,
+          os.path.join(CSRC, "cli", "msd_compare.cpp"), os.path.join(nn_dir, "npy.cpp"), "-o", CLI_COMPARE])
+    return CLI_COMPARE
+
+
 def build_all(verbose=True):
     built = [build_hip()]
     nn = build_nn()
     if nn:
         built.append(nn)
+    built.append(build_cli())
     if verbose:
         for b in built:
             print("built", b)

@@ -63,7 +63,7 @@ hipError_t get_scratch(hipStream_t stream, GnScratch *out) {
     return hipSuccess;
 }
 
-Tuning g_tuning = {0, 0, 0, 0, 0, 0};
+Tuning g_tuning = {0, 0, 0, 0, 0, 0, 0};
 
 }  // namespace msd
 
@@ -145,6 +145,10 @@ int msd_set_tuning(int knob, int value) {
         case MSD_TUNE_ACT_VECTORS:
             if (value && value != 1 && value != 2 && value != 4) return MSD_ERR_INVALID_VALUE;
             g_tuning.act_vectors = value;
+            return MSD_OK;
+        case MSD_TUNE_SOFTMAX_ROWS:
+            if (value && value != 16 && value != 32 && value != 64) return MSD_ERR_INVALID_VALUE;
+            g_tuning.softmax_rows = value;
             return MSD_OK;
         default:
             return MSD_ERR_INVALID_VALUE;

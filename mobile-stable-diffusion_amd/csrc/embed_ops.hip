@@ -1,5 +1,5 @@
 // Neighbours of the norm / activation path for gfx950: the Linear layers that act on
-// the few rows of the time embedding (weight-streaming, one output column per
+// the few rows of the time embedding (weight-streaming, one or two output columns per
 // wavefront), the row softmax of the attention blocks (a row held in the registers
 // of a team of lanes) and the DDIM latent update.
 #include "msd_device.h"
@@ -12,77 +12,87 @@ namespace {
 
 // ---------------------------------------------------------------------------
 // y[m, n] = act_out(act_in(x)[m, k] . w[n, k]^T + bias[n]) for m <= 8 rows.
-// The time is the single pass over w (n*k elements); x is staged once per workgroup
-// in LDS as float with act_in already applied.  A wavefront owns one column: lane l
-// multiplies 16-byte pieces l, l+64, ... of the weight row, every load of a round of
-// UN pieces issued before the first use, then the M partial sums go through the DPP
-// tree.  Each lane adds its pieces in ascending k; the tree order is fixed, so the
-// result does not depend on the launch shape.
+// The time is the single pass over w (n*k elements) plus launch and memory latency, so
+// the kernel is built to have one latency, not two in a row: a workgroup is a single
+// wavefront that owns CPW columns; lane l requests 16-byte pieces l, l+64, ... of its
+// weight rows and the same pieces of every x row (a few KiB that every wavefront
+// reads from cache) before it uses any of them.  No LDS, no barrier.  With SiLU on the
+// input each lane activates its own x pieces, and two columns share that work.
+// Each lane adds its pieces in ascending k, then the M x CPW partial sums go through
+// the DPP tree, so the result does not depend on the launch shape.
 // ---------------------------------------------------------------------------
-constexpr int kLinThreads = 256;
-constexpr int kLinWaves = kLinThreads / kWave;
-constexpr int kLinRound = 4;            // 16-byte weight loads in flight per lane
-constexpr size_t kLinMaxStaged = 12288; // floats of x in LDS (48 KiB)
 
-template <typename T, int M>
-__global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(
+template <typename T, int M, int CPW>
+__global__ __launch_bounds__(kWave) void linear_rows_kernel(
     const T *__restrict__ x, const T *__restrict__ w, const float *__restrict__ bias,
     T *__restrict__ y, uint32_t m, uint32_t n, uint32_t kvecs, int act_in, int act_out) {
     constexpr int EPV = Store<T>::EPV;
-    extern __shared__ float xs[];  // [M][kvecs * EPV]
-    const uint32_t k = kvecs * EPV;
+    // pieces per lane per round: one round covers k = 2048 (float with more than 4 rows: 1024)
+    constexpr int kLinRound = (sizeof(T) == 4 && M <= 4) ? 8 : 4;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t col0 = blockIdx.x * CPW;
     const u32x4 *xin = reinterpret_cast<const u32x4 *>(x);
-    for (uint32_t v = threadIdx.x; v < M * kvecs; v += kLinThreads) {
-        const uint32_t row = v / kvecs, piece = v - row * kvecs;
-        float f[EPV];
-        Store<T>::unpack(xin[(size_t)min(row, m - 1) * kvecs + piece], f);  // rows >= m repeat the last
-        if (act_in) {
+    const u32x4 *win = reinterpret_cast<const u32x4 *>(w);
+    float acc[CPW][M];
 #pragma unroll
-            for (int e = 0; e < EPV; e++) f[e] = silu_f(f[e]);
-        }
+    for (int c = 0; c < CPW; c++)
 #pragma unroll
-        for (int e = 0; e < EPV; e++) xs[row * k + piece * EPV + e] = f[e];
-    }
-    __syncthreads();
-    const uint32_t lane = threadIdx.x & (kWave - 1);
-    const uint32_t col = blockIdx.x * kLinWaves + threadIdx.x / kWave;
-    if (col >= n) return;  // whole wavefront; no barrier follows
-    const u32x4 *wrow = reinterpret_cast<const u32x4 *>(w) + (size_t)col * kvecs;
-    float acc[M];
-#pragma unroll
-    for (int i = 0; i < M; i++) acc[i] = 0.0f;
+        for (int i = 0; i < M; i++) acc[c][i] = 0.0f;
     for (uint32_t base = lane; base < kvecs; base += kWave * kLinRound) {
-        u32x4 raw[kLinRound];
-#pragma unroll
-        for (int u = 0; u < kLinRound; u++)
-            raw[u] = load_stream(wrow + min(base + u * kWave, kvecs - 1));
+        u32x4 wraw[CPW][kLinRound], xraw[M][kLinRound];
 #pragma unroll
         for (int u = 0; u < kLinRound; u++) {
-            const uint32_t piece = base + u * kWave;
-            if (piece < kvecs) {
-                float wf[EPV];
-                Store<T>::unpack(raw[u], wf);
+            const uint32_t piece = min(base + u * kWave, kvecs - 1);
+#pragma unroll
+            for (int c = 0; c < CPW; c++)  // a column past the last re-reads the last one
+                wraw[c][u] = load_stream(win + (size_t)min(col0 + c, n - 1) * kvecs + piece);
+#pragma unroll
+            for (int i = 0; i < M; i++)    // rows >= m repeat the last row
+                xraw[i][u] = xin[(size_t)min((uint32_t)i, m - 1) * kvecs + piece];
+        }
+#pragma unroll
+        for (int u = 0; u < kLinRound; u++) {
+            if (base + u * kWave < kvecs) {
+                float xf[M][EPV];
 #pragma unroll
                 for (int i = 0; i < M; i++) {
-                    const float *xr = xs + i * k + piece * EPV;
+                    Store<T>::unpack(xraw[i][u], xf[i]);
+                    if (act_in) {
 #pragma unroll
-                    for (int e = 0; e < EPV; e++) acc[i] = fmaf(xr[e], wf[e], acc[i]);
+                        for (int e = 0; e < EPV; e++) xf[i][e] = silu_f(xf[i][e]);
+                    }
+                }
+#pragma unroll
+                for (int c = 0; c < CPW; c++) {
+                    float wf[EPV];
+                    Store<T>::unpack(wraw[c][u], wf);
+#pragma unroll
+                    for (int i = 0; i < M; i++)
+#pragma unroll
+                        for (int e = 0; e < EPV; e++) acc[c][i] = fmaf(xf[i][e], wf[e], acc[c][i]);
                 }
             }
         }
     }
-    float mine = 0.0f;
 #pragma unroll
-    for (int i = 0; i < M; i++) {
-        const float total = wave_sum(acc[i]);
-        if (lane == (uint32_t)i) mine = total;
-    }
-    if (lane < m) {
-        float r = mine + (bias != nullptr ? bias[col] : 0.0f);
-        if (act_out) r = silu_f(r);
-        Store<T>::store1(y + (size_t)lane * n + col, r);
+    for (int c = 0; c < CPW; c++) {
+        float mine = 0.0f;
+#pragma unroll
+        for (int i = 0; i < M; i++) {
+            const float total = wave_sum(acc[c][i]);
+            if (lane == (uint32_t)i) mine = total;
+        }
+        const uint32_t col = col0 + c;
+        if (lane < m && col < n) {
+            float r = mine + (bias != nullptr ? bias[col] : 0.0f);
+            if (act_out) r = silu_f(r);
+            Store<T>::store1(y + (size_t)lane * n + col, r);
+        }
     }
 }
+
+constexpr int kLinThreads = 256;  // workgroup of the scalar kernel below
+constexpr int kLinWaves = kLinThreads / kWave;
 
 // Any k / alignment: x is read from global memory (it is a few KiB and stays cached).
 template <typename T>
@@ -242,6 +252,92 @@ __global__ __launch_bounds__(kSmThreads) void softmax_short_kernel(const T *x, T
     }
 }
 
+// Short rows whose length is not a multiple of a 16-byte vector (77 text tokens): a
+// workgroup takes RB consecutive rows (RB a multiple of 8) as one flat, 16-byte aligned
+// run of memory (such a block is a whole number of vectors for any row length), moves it
+// through LDS with full vectors, and a team of 4 lanes per row does the arithmetic on
+// the LDS copy.
+constexpr int kSmFlatTeam = 4;
+constexpr uint32_t kSmFlatMaxCols = 128;  // RB = 64: 32 KiB of LDS
+
+template <typename T, int RB, int ITERS>
+__global__ __launch_bounds__(RB * kSmFlatTeam) void softmax_flat_kernel(const T *x, T *y, uint32_t cols,
+                                                                       int stable) {
+    constexpr int EPV = Store<T>::EPV;
+    constexpr int NT = RB * kSmFlatTeam;
+    constexpr int UN = 4;
+    extern __shared__ float tile[];  // [RB][cols], cols <= ITERS * kSmFlatTeam
+    const uint32_t block_vecs = RB * cols / EPV;
+    const size_t first = (size_t)blockIdx.x * block_vecs;
+    const u32x4 *in = reinterpret_cast<const u32x4 *>(x) + first;
+    u32x4 *out = reinterpret_cast<u32x4 *>(y) + first;
+    for (uint32_t base = threadIdx.x; base < block_vecs; base += NT * UN) {
+        u32x4 raw[UN];
+#pragma unroll
+        for (int u = 0; u < UN; u++) raw[u] = load_stream(in + min(base + u * NT, block_vecs - 1));
+#pragma unroll
+        for (int u = 0; u < UN; u++) {
+            const uint32_t v = base + u * NT;
+            if (v < block_vecs) {
+                float f[EPV];
+                Store<T>::unpack(raw[u], f);
+#pragma unroll
+                for (int e = 0; e < EPV; e++) tile[v * EPV + e] = f[e];
+            }
+        }
+    }
+    __syncthreads();
+    // the lane's share of its row, from LDS into registers with independent reads
+    float *row = tile + (threadIdx.x / kSmFlatTeam) * cols;
+    const uint32_t j = threadIdx.x % kSmFlatTeam;
+    float f[ITERS];
+    float mx = kNegInf;
+#pragma unroll
+    for (int i = 0; i < ITERS; i++) {
+        const uint32_t c = j + i * kSmFlatTeam;
+        f[i] = c < cols ? row[c] : kNegInf;
+        mx = fmaxf(mx, f[i]);
+    }
+    float shift = 0.0f;
+    if (stable) {
+        mx = team_max<kSmFlatTeam>(mx);
+        shift = mx == kNegInf ? 0.0f : mx;
+    }
+    const float bias = -shift * kLog2e;
+    float total = 0.0f;
+#pragma unroll
+    for (int i = 0; i < ITERS; i++) {
+        f[i] = __builtin_amdgcn_exp2f(fmaf(f[i], kLog2e, bias));
+        total += f[i];
+    }
+    total = team_sum<kSmFlatTeam>(total);
+    const float inv = 1.0f / total;
+#pragma unroll
+    for (int i = 0; i < ITERS; i++) {
+        const uint32_t c = j + i * kSmFlatTeam;
+        if (c < cols) row[c] = f[i] * inv;
+    }
+    __syncthreads();
+    for (uint32_t v = threadIdx.x; v < block_vecs; v += NT) {
+        float g[EPV];
+#pragma unroll
+        for (int e = 0; e < EPV; e++) g[e] = tile[v * EPV + e];
+        store_stream(out + v, Store<T>::pack(g));
+    }
+}
+
+template <typename T, int ITERS>
+void softmax_flat_launch(const T *x, T *y, uint32_t blocks, uint32_t rb, uint32_t cols, int stable,
+                         hipStream_t stream) {
+    const size_t lds = (size_t)rb * cols * sizeof(float);
+    if (rb == 64)
+        hipLaunchKernelGGL((softmax_flat_kernel<T, 64, ITERS>), dim3(blocks), dim3(256), lds, stream, x, y, cols, stable);
+    else if (rb == 32)
+        hipLaunchKernelGGL((softmax_flat_kernel<T, 32, ITERS>), dim3(blocks), dim3(128), lds, stream, x, y, cols, stable);
+    else
+        hipLaunchKernelGGL((softmax_flat_kernel<T, 16, ITERS>), dim3(blocks), dim3(64), lds, stream, x, y, cols, stable);
+}
+
 // ---------------------------------------------------------------------------
 // DDIM update (eta = 0): the three float loops of the replaced host code as one pass,
 // with individually rounded operations in the same order, so float32 storage gives
@@ -290,10 +386,12 @@ template <typename T, int M>
 void linear_launch(const T *x, const T *w, const float *bias, T *y, uint32_t m, uint32_t n, uint32_t k,
                    int act_in, int act_out, hipStream_t stream) {
     constexpr int EPV = Store<T>::EPV;
-    const uint32_t blocks = (n + kLinWaves - 1) / kLinWaves;
-    hipLaunchKernelGGL((linear_rows_kernel<T, M>), dim3(blocks), dim3(kLinThreads),
-                       (size_t)M * k * sizeof(float), stream, x, w, bias, y, m, n, k / EPV, act_in,
-                       act_out);
+    if (act_in)  // two columns per wavefront share the activated x
+        hipLaunchKernelGGL((linear_rows_kernel<T, M, 2>), dim3((n + 1) / 2), dim3(kWave), 0, stream, x, w, bias,
+                           y, m, n, k / EPV, act_in, act_out);
+    else
+        hipLaunchKernelGGL((linear_rows_kernel<T, M, 1>), dim3(n), dim3(kWave), 0, stream, x, w, bias, y, m, n,
+                           k / EPV, act_in, act_out);
 }
 
 template <typename T, int VPL, int TL>
@@ -314,11 +412,10 @@ int linear_rows_dispatch(const void *xv, const void *wv, const float *bias, void
     const T *w = static_cast<const T *>(wv);
     T *y = static_cast<T *>(yv);
     if (m == 0 || n == 0) return MSD_OK;
-    if (m > 8 || n > 0x7FFFFFFFull / kLinWaves || k > 0x7FFFFFFFull) return MSD_ERR_INVALID_VALUE;
+    if (m > 8 || n > 0x7FFFFFFFull || k > 0x7FFFFFFFull) return MSD_ERR_INVALID_VALUE;
     const uint32_t m_pad = m <= 1 ? 1 : m <= 2 ? 2 : m <= 4 ? 4 : 8;
-    const bool staged = k != 0 && k % EPV == 0 && aligned16(x) && aligned16(w) &&
-                        (size_t)m_pad * k <= kLinMaxStaged;
-    if (staged) {
+    const bool vectors = k != 0 && k % EPV == 0 && aligned16(x) && aligned16(w);
+    if (vectors) {
         switch (m_pad) {
             case 1: linear_launch<T, 1>(x, w, bias, y, (uint32_t)m, (uint32_t)n, (uint32_t)k, act_in, act_out, stream); break;
             case 2: linear_launch<T, 2>(x, w, bias, y, (uint32_t)m, (uint32_t)n, (uint32_t)k, act_in, act_out, stream); break;
@@ -356,13 +453,30 @@ int softmax_dispatch(const void *xv, void *yv, size_t rows, size_t cols, int sta
         else softmax_team_launch<T, 16, 64>(x, y, r, rv, stable, stream);
         return launch_status();
     }
+    // The flat kernel pays two LDS round trips per row; it wins once the launch is large
+    // enough for the row-per-wavefront kernel to be bound by its 2-byte accesses
+    // (measured crossover near 20000 rows of 77).  A set knob forces it for any size.
+    const uint32_t rb = g_tuning.softmax_rows ? (uint32_t)g_tuning.softmax_rows : 64u;
+    const bool flat_pays = g_tuning.softmax_rows ? rows >= rb : rows >= 24576;
+    if (cols <= kSmFlatMaxCols && cols >= 8 && flat_pays && aligned16(x) && aligned16(y)) {
+        // whole blocks of rb rows through the flat kernel, the rest (if any) row by row below
+        const uint32_t blocks = r / rb;
+        if (c <= 20 * kSmFlatTeam) softmax_flat_launch<T, 20>(x, y, blocks, rb, c, stable, stream);
+        else softmax_flat_launch<T, 32>(x, y, blocks, rb, c, stable, stream);
+        const uint32_t done = blocks * rb;
+        if (done == r) return launch_status();
+        x += (size_t)done * c;
+        y += (size_t)done * c;
+        rows -= done;
+    }
+    const uint32_t r_left = (uint32_t)rows;
     const dim3 grid((uint32_t)((rows + waves_per_block - 1) / waves_per_block));
     if (cols <= 2 * kWave)
-        hipLaunchKernelGGL((softmax_short_kernel<T, 2>), grid, dim3(kSmThreads), 0, stream, x, y, r, c, stable);
+        hipLaunchKernelGGL((softmax_short_kernel<T, 2>), grid, dim3(kSmThreads), 0, stream, x, y, r_left, c, stable);
     else if (cols <= 8 * kWave)
-        hipLaunchKernelGGL((softmax_short_kernel<T, 8>), grid, dim3(kSmThreads), 0, stream, x, y, r, c, stable);
+        hipLaunchKernelGGL((softmax_short_kernel<T, 8>), grid, dim3(kSmThreads), 0, stream, x, y, r_left, c, stable);
     else
-        hipLaunchKernelGGL((softmax_generic_kernel<T>), grid, dim3(kSmThreads), 0, stream, x, y, r, c, stable);
+        hipLaunchKernelGGL((softmax_generic_kernel<T>), grid, dim3(kSmThreads), 0, stream, x, y, r_left, c, stable);
     return launch_status();
 }
 

@@ -35,6 +35,7 @@ struct Tuning {
     int ln_threads;
     int geglu_vectors;
     int act_vectors;
+    int softmax_rows;
 };
 extern Tuning g_tuning;
 

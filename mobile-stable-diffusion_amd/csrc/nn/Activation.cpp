@@ -44,4 +44,13 @@ int permute3D_0_2_1(hipStream_t stream, const DeviceBuffer &src, DeviceBuffer &d
     return msd_permute_0_2_1(src.ptr(), dst.ptr(), isize, jsize, ksize, (int)src.dtype(), stream);
 }
 
+int softmax(hipStream_t stream, const DeviceBuffer &src, DeviceBuffer &dst, size_t chunkSize, bool stable) {
+    if (dst.bytes() != src.bytes() || dst.dtype() != src.dtype())
+        throw std::runtime_error("dst size / type != src size / type");
+    if (chunkSize == 0 || src.count() % chunkSize != 0)
+        throw std::runtime_error("element count % chunkSize != 0");
+    return msd_softmax(src.ptr(), dst.ptr(), src.count() / chunkSize, chunkSize, stable ? 1 : 0,
+                       (int)src.dtype(), stream);
+}
+
 }  // namespace msd

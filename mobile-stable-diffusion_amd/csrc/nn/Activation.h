@@ -27,4 +27,12 @@ int chunkwise_add(hipStream_t stream, const DeviceBuffer &a, const DeviceBuffer 
 int permute3D_0_2_1(hipStream_t stream, const DeviceBuffer &src, DeviceBuffer &dst, size_t isize,
                     size_t jsize, size_t ksize);
 
+// Row softmax in chunks of chunkSize elements: utilKernel->softmax (K/util.cl:150-187) as the
+// attention blocks enqueue it, in place, one workgroup per chunk
+// (M/nn/CrossAttention.cpp:362-377, M/nn/AttnBlock.cpp:196-206).  stable = false is that
+// kernel's exp(x) / sum; true subtracts the chunk maximum first.  Throws std::runtime_error
+// when the element count is not a multiple of chunkSize.
+int softmax(hipStream_t stream, const DeviceBuffer &src, DeviceBuffer &dst, size_t chunkSize,
+            bool stable = false);
+
 }  // namespace msd

@@ -11,8 +11,10 @@
 
 #include "Activation.h"
 #include "GEGLU.h"
+#include "DDIMSampler.h"
 #include "GroupNorm.h"
 #include "LayerNorm.h"
+#include "Linear.h"
 #include "TimestepEmbedding.h"
 #include "UNetNormActStep.h"
 #include "util.h"
@@ -195,6 +197,78 @@ int msdnn_ddim_timesteps(int steps, int *out, int cap) {
         return 0;
     });
     return rc < 0 ? rc : n;
+}
+
+// ---- Linear on embedding rows; weights from .npy names (init) or from host arrays (init_from)
+void *msdnn_linear_create(void *stream, size_t in_features, size_t out_features, const char *weight_name,
+                          const char *bias_name, int dtype) {
+    Linear *l = nullptr;
+    guarded([&] {
+        l = new Linear(static_cast<hipStream_t>(stream), in_features, out_features, weight_name ? weight_name : "",
+                       bias_name ? bias_name : "", dtype == MSD_DTYPE_F16 ? DType::F16 : DType::F32);
+        return 0;
+    });
+    return l;
+}
+int msdnn_linear_init(void *h) {
+    return guarded([&] {
+        static_cast<Linear *>(h)->init();
+        return 0;
+    });
+}
+int msdnn_linear_init_from(void *h, const float *weight, size_t weight_count, const float *bias,
+                           size_t bias_count) {
+    return guarded([&] {
+        static_cast<Linear *>(h)->init(std::vector<float>(weight, weight + weight_count),
+                                       bias ? std::vector<float>(bias, bias + bias_count) : std::vector<float>());
+        return 0;
+    });
+}
+int msdnn_linear_forward(void *h, void *in, size_t in_bytes, void *out, size_t out_bytes, int dtype,
+                         int silu_on_input, int silu_on_output) {
+    return guarded([&] {
+        DeviceBuffer i = wrap(in, in_bytes, dtype), o = wrap(out, out_bytes, dtype);
+        return static_cast<Linear *>(h)->forwardSilu(i, o, silu_on_input != 0, silu_on_output != 0);
+    });
+}
+void msdnn_linear_destroy(void *h) { delete static_cast<Linear *>(h); }
+
+// ---- row softmax
+int msdnn_softmax(void *stream, void *src, void *dst, size_t bytes, int dtype, size_t chunk_size, int stable) {
+    return guarded([&] {
+        DeviceBuffer s = wrap(src, bytes, dtype), d = wrap(dst, bytes, dtype);
+        return softmax(static_cast<hipStream_t>(stream), s, d, chunk_size, stable != 0);
+    });
+}
+
+// ---- DDIM sampler.  The noise model is a C callback: model(x, t, e_t, bytes, user) fills e_t for
+// latent x on the sampler's stream and returns 0.  x_T (device, `bytes` long) is not modified;
+// the final latent is copied to `out` (device, same size).
+typedef int (*msdnn_model_fn)(void *x, int t, void *e_t, size_t bytes, void *user);
+int msdnn_ddim_sample(void *stream, void *x_T, size_t bytes, int dtype, int steps, msdnn_model_fn model,
+                      void *user, void *out) {
+    return guarded([&] {
+        hipStream_t st = static_cast<hipStream_t>(stream);
+        DDIMSampler sampler(st, [&](const DeviceBuffer &x, int t, const DeviceBuffer &, DeviceBuffer &e_t) {
+            return model(x.ptr(), t, e_t.ptr(), x.bytes(), user);
+        });
+        DeviceBuffer start = wrap(x_T, bytes, dtype), none;
+        const int shape[3] = {0, 0, 0};
+        DeviceBuffer img = sampler.sample(&start, steps, shape, none);
+        return (int)hipMemcpy(out, img.ptr(), bytes, hipMemcpyDeviceToDevice);
+    });
+}
+// make_schedule through the sampler object: alphas / alphas_prev for a timestep list
+int msdnn_ddim_make_schedule(const int *timesteps, int count, float *alphas, float *alphas_prev) {
+    return guarded([&] {
+        DDIMSampler sampler(nullptr, DDIMSampler::ApplyModel());
+        const auto s = sampler.make_schedule(std::vector<int>(timesteps, timesteps + count));
+        for (int i = 0; i < count; i++) {
+            alphas[i] = s.first[(size_t)i];
+            alphas_prev[i] = s.second[(size_t)i];
+        }
+        return 0;
+    });
 }
 
 // ---- golden-file comparison (util::testBuffer)

@@ -193,3 +193,114 @@ def test_step_runner_eager_and_graph(msd, nn, cuda):
     assert nn.msdnn_step_run(st0, 1, 0, (ctypes.c_long * 1)(5), 1) == 0
     torch.cuda.synchronize()
     nn.msdnn_step_destroy(st0)
+
+
+# ----------------------------------------------------------------- neighbours of the path
+@pytest.mark.parametrize("half", [False, True], ids=["f32", "f16"])
+def test_linear_objects_run_the_time_embedding_mlp(msd, nn, orc, cuda, tmp_path, half):
+    """time_embed_0 + SiLU, time_embed_2, then a ResBlock's SiLU + embed_linear, weights from .npy."""
+    import torch
+    shapes = {"time_embed_0": (1280, 320), "time_embed_2": (1280, 1280), "embed_linear": (640, 1280)}
+    weights = {}
+    for i, (name, (n, k)) in enumerate(shapes.items()):
+        w = orc.normal((n, k), seed=300 + i, sigma=k ** -0.5)
+        b = orc.normal((n,), seed=310 + i, sigma=0.1)
+        np.save(tmp_path / (name + "_weight.npy"), w)
+        np.save(tmp_path / (name + "_bias.npy"), b)
+        weights[name] = (orc.round_to_half(w) if half else w, b)
+    temb = np.stack([orc.timestep_embedding(t) for t in (981, 21)])
+    temb = orc.round_to_half(temb) if half else temb
+    rnd = orc.round_to_half if half else (lambda v: v)
+    h = rnd(orc.silu(orc.linear(temb, *weights["time_embed_0"])))
+    emb = rnd(orc.linear(h, *weights["time_embed_2"]))
+    ref = rnd(orc.linear(orc.silu(emb), *weights["embed_linear"]))
+
+    layers = {}
+    for name, (n, k) in shapes.items():
+        l = nn.msdnn_linear_create(None, k, n, (name + "_weight.npy").encode(), (name + "_bias.npy").encode(),
+                                   int(half))
+        assert l and nn.msdnn_linear_init(l) == 0, msd.nn_last_error()
+        layers[name] = l
+    dt = torch.float16 if half else torch.float32
+    es = 2 if half else 4
+    x = _dev(temb, cuda, half)
+    hd = torch.empty((2, 1280), dtype=dt, device=cuda)
+    ed = torch.empty((2, 1280), dtype=dt, device=cuda)
+    od = torch.empty((2, 640), dtype=dt, device=cuda)
+    fw = nn.msdnn_linear_forward
+    assert fw(layers["time_embed_0"], _ptr(x), 2 * 320 * es, _ptr(hd), 2 * 1280 * es, int(half), 0, 1) == 0
+    assert fw(layers["time_embed_2"], _ptr(hd), 2 * 1280 * es, _ptr(ed), 2 * 1280 * es, int(half), 0, 0) == 0
+    assert fw(layers["embed_linear"], _ptr(ed), 2 * 1280 * es, _ptr(od), 2 * 640 * es, int(half), 1, 0) == 0
+    if half:
+        # three layers deep: an fp16 rounding flip upstream moves the result by a few ulps
+        np.testing.assert_allclose(od.float().cpu().numpy(), ref, atol=4e-3, rtol=2e-3)
+        assert_close_f16(ed.float().cpu().numpy(), emb, "time_embed f16")
+    else:
+        assert_close_f32(ed.cpu().numpy(), emb, what="time_embed")
+        assert_close_f32(od.cpu().numpy(), ref, what="embed_linear")
+    # the reference's refusals (M/nn/Linear.cpp:78-92)
+    assert fw(layers["time_embed_2"], _ptr(hd), 2 * 1280 * es, _ptr(hd), 2 * 1280 * es, int(half), 0, 0) < 0
+    assert msd.nn_last_error() == "Linear not support input == output"
+    assert fw(layers["time_embed_2"], _ptr(hd), (2 * 1280 - 1) * es, _ptr(ed), 2 * 1280 * es, int(half), 0, 0) < 0
+    assert msd.nn_last_error() == "inputSize % weightShape[1] != 0"
+    many = torch.zeros((9, 1280), dtype=dt, device=cuda)
+    out9 = torch.zeros((9, 1280), dtype=dt, device=cuda)
+    assert fw(layers["time_embed_2"], _ptr(many), 9 * 1280 * es, _ptr(out9), 9 * 1280 * es, int(half), 0, 0) < 0
+    for l in layers.values():
+        nn.msdnn_linear_destroy(l)
+
+
+def test_softmax_function_in_place_like_cross_attention(msd, nn, orc, cuda):
+    x = orc.normal((8 * 64, 77), seed=400, sigma=2.0)
+    xd = _dev(x, cuda)
+    assert nn.msdnn_softmax(None, _ptr(xd), _ptr(xd), x.size * 4, 0, 77, 0) == 0, msd.nn_last_error()
+    assert_close_f32(xd.cpu().numpy(), orc.softmax(x), what="softmax object")
+    assert nn.msdnn_softmax(None, _ptr(xd), _ptr(xd), x.size * 4, 0, 76, 0) < 0
+    assert msd.nn_last_error() == "element count % chunkSize != 0"
+
+
+def test_ddim_sampler_object_walks_the_schedule_from_the_back(msd, nn, orc, cuda):
+    """sample() with a stand-in noise model given as a callback; bit-exact against the oracle."""
+    import torch
+    n = 4 * 32 * 32
+    x0 = orc.normal((n,), seed=500)
+    noise = orc.normal((n,), seed=501)
+    nd = _dev(noise, cuda)
+    seen = []
+
+    def model(x_ptr, t, e_ptr, nbytes, user):
+        # e_t = 0.5 * x + (0.25 + 0.001 t) * noise, written into the sampler's e_t buffer
+        seen.append(t)
+        scale = float(np.float32(0.25 + 0.001 * t))
+        e = cur["x"] * 0.5 + nd * scale
+        msd.check(msd.load_library().msd_copy(_ptr(e), ctypes.c_void_p(e_ptr), nbytes, None))
+        cur["e"] = e  # keep alive until the stream has consumed it
+        return 0
+
+    # the sampler updates its own copy of x in place; mirror it in a tensor the model can read
+    steps = 25
+    ts, a, ap, s1m = orc.ddim_schedule(steps)
+    x = x0.copy()
+    for index in range(len(ts) - 1, -1, -1):
+        scale = np.float32(0.25 + 0.001 * ts[index])
+        e = (np.float32(0.5) * x + scale * noise).astype(np.float32)
+        x = orc.ddim_update(x, e, a[index], ap[index], s1m[index])
+
+    xd = _dev(x0, cuda)
+    out = torch.empty_like(xd)
+    cur = {}
+
+    def model_reading_sampler_memory(x_ptr, t, e_ptr, nbytes, user):
+        # wrap the sampler's latent: copy it into a torch tensor first
+        view = torch.empty(n, dtype=torch.float32, device=cuda)
+        msd.check(msd.load_library().msd_copy(ctypes.c_void_p(x_ptr), _ptr(view), nbytes, None))
+        cur["x"] = view
+        return model(x_ptr, t, e_ptr, nbytes, user)
+
+    cb = msd.MODEL_FN(model_reading_sampler_memory)
+    rc = nn.msdnn_ddim_sample(None, _ptr(xd), n * 4, 0, steps, cb, None, _ptr(out))
+    assert rc == 0, msd.nn_last_error()
+    assert seen == [int(v) for v in ts[::-1]]  # 961, 921, ..., 1
+    assert np.array_equal(xd.cpu().numpy(), x0)  # x_T untouched
+    assert np.array_equal(out.cpu().numpy(), x)
+    assert nn.msdnn_ddim_sample(None, _ptr(xd), n * 4, 0, 501, cb, None, _ptr(out)) < 0

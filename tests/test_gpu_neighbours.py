@@ -156,11 +156,33 @@ def test_softmax_attention_shapes(msd, orc, cuda, rows, cols, stable, half):
 
 
 @pytest.mark.parametrize("rows,cols", [(1, 1), (3, 4), (5, 8), (9, 40), (7, 300), (4, 600), (6, 1000),
-                                       (3, 2048), (5, 8192), (2, 10000), (33, 129), (2, 513)])
+                                       (3, 2048), (5, 8192), (2, 10000), (33, 129), (2, 513),
+                                       (200, 100), (128, 9), (64, 128), (191, 127), (70, 8)])
 def test_softmax_edge_shapes(msd, orc, cuda, rows, cols):
     for half in (False, True):
         for stable in (0, 1):
             _softmax_case(msd, orc, cuda, rows, cols, 8100 + cols, half, stable, sigma=1.5)
+
+
+@pytest.mark.parametrize("rb", [16, 32, 64])
+def test_softmax_short_rows_flat_kernel(msd, orc, cuda, rb):
+    """Rows of 77 / 100 moved as flat 16-byte vectors, rb rows per workgroup, plus a ragged tail."""
+    lib = msd.load_library()
+    assert lib.msd_set_tuning(msd.TUNE_SOFTMAX_ROWS, rb) == 0
+    try:
+        for rows, cols in [(rb * 5 + 3, 77), (rb, 100), (2 * rb + 1, 9), (rb * 3, 127)]:
+            for half in (False, True):
+                for stable in (0, 1):
+                    _softmax_case(msd, orc, cuda, rows, cols, 8300 + cols + rb, half, stable, inplace=True)
+    finally:
+        assert lib.msd_set_tuning(msd.TUNE_SOFTMAX_ROWS, 0) == 0
+    assert lib.msd_set_tuning(msd.TUNE_SOFTMAX_ROWS, 48) == 1
+
+
+def test_softmax_cross_attention_full_rows(msd, orc, cuda):
+    """All 2 x 8 x 4096 query rows against 77 text tokens (the size that takes the flat kernel)."""
+    _softmax_case(msd, orc, cuda, 2 * 8 * 4096, 77, 8400, True, 0, inplace=True)
+    _softmax_case(msd, orc, cuda, 2 * 8 * 4096 + 5, 77, 8401, False, 1)
 
 
 def test_softmax_overflow_follows_the_reference_unless_stable(msd, orc, cuda):

@@ -135,3 +135,35 @@ def test_ddim_through_host_layer(msd, nn, orc):
         n = nn.msdnn_ddim_timesteps(steps, buf, 1000)
         assert list(buf[:n]) == orc.ddim_timesteps(steps)
     assert nn.msdnn_ddim_timesteps(0, buf, 1000) < 0
+
+
+def test_linear_preconditions(msd, nn, tmp_path):
+    np.save(tmp_path / "w_1280x320.npy", np.zeros((1280, 320), dtype=np.float32))
+    np.save(tmp_path / "b_1280.npy", np.zeros(1280, dtype=np.float32))
+    np.save(tmp_path / "b_320.npy", np.zeros(320, dtype=np.float32))
+    lin = nn.msdnn_linear_create(None, 320, 640, b"w_1280x320.npy", b"b_1280.npy", 0)
+    assert nn.msdnn_linear_init(lin) < 0
+    assert msd.nn_last_error() == "weight.num_vals != (weightShape[0] * weightShape[1])"  # M/nn/Linear.cpp:53-59
+    nn.msdnn_linear_destroy(lin)
+    lin = nn.msdnn_linear_create(None, 320, 1280, b"w_1280x320.npy", b"b_320.npy", 0)
+    assert nn.msdnn_linear_init(lin) < 0
+    assert msd.nn_last_error() == "bias.num_vals != weightShape[0]"  # M/nn/Linear.cpp:62-70
+    nn.msdnn_linear_destroy(lin)
+    lin = nn.msdnn_linear_create(None, 320, 1280, b"missing.npy", b"", 0)
+    assert nn.msdnn_linear_init(lin) < 0 and "Unable to open file" in msd.nn_last_error()
+    # forward before init
+    assert nn.msdnn_linear_forward(lin, None, 0, None, 0, 0, 0, 0) < 0
+    assert msd.nn_last_error() == "Linear: init() not called"
+    nn.msdnn_linear_destroy(lin)
+
+
+def test_ddim_make_schedule_through_sampler_object(msd, nn, orc):
+    ts, a, ap, _ = orc.ddim_schedule(50)
+    n = len(ts)
+    t_arr = (ctypes.c_int * n)(*[int(v) for v in ts])
+    ga, gp = (ctypes.c_float * n)(), (ctypes.c_float * n)()
+    assert nn.msdnn_ddim_make_schedule(t_arr, n, ga, gp) == 0, msd.nn_last_error()
+    assert np.array_equal(np.array(ga[:], dtype=np.float32), a)
+    assert np.array_equal(np.array(gp[:], dtype=np.float32), ap)
+    bad = (ctypes.c_int * 1)(1000)
+    assert nn.msdnn_ddim_make_schedule(bad, 1, ga, gp) < 0  # the reference would read past its table
