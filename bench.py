@@ -464,7 +464,7 @@ def neighbour_table(torch, msd, dev, stream):
     return rows
 
 
-def cpu_baseline(total_bytes, budget_s=12.0):
+def cpu_baseline(total_bytes, budget_s=24.0):
     """The reference path as host loops (the CPU oracle, fp32, unfused passes exactly as the
     reference enqueues them) over the layers of one full step, timed on this host's cores.
     Every layer runs `reps` times on its own input (reps sized so the whole leg takes about
