@@ -8,7 +8,7 @@ each layer on its own HBM-resident buffers, launched back to back on one stream.
 `value` = algorithmic bytes of one step / time per step.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode graph|eager]
-                    [--no-cpu] [--no-shapes]
+                    [--no-cpu] [--no-shapes] [--tables shapes,fusions,neighbours]
 
 Prints ONE JSON line (see the keys below).  The CPU oracle is used only for the
 `cpu_baseline` leg.
@@ -529,7 +529,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--mode", choices=["graph", "eager"], default="graph")
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--no-shapes", action="store_true")
+    ap.add_argument("--no-shapes", action="store_true", help="skip the per-kernel tables")
+    ap.add_argument("--tables", default="shapes,fusions,neighbours",
+                    help="comma list of the per-kernel tables to measure")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="for rocprofv3 --pmc runs: one 64 MiB device copy (known traffic) then three "
                          "eager steps; prints nothing")
@@ -618,9 +620,12 @@ def main():
         "roofline": roofline,
         "kernel_families": families,
     }
-    if not args.no_shapes:
+    tables = set() if args.no_shapes else set(t for t in args.tables.split(",") if t)
+    if "shapes" in tables:
         out["shapes"] = shape_table(torch, msd, dev, stream)
+    if "fusions" in tables:
         out["fusions"] = fusion_table(torch, msd, dev, stream)
+    if "neighbours" in tables:
         out["neighbours"] = neighbour_table(torch, msd, dev, stream)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(step.bytes)
