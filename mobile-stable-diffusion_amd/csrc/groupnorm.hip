@@ -123,6 +123,9 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
                                         uint32_t v_begin, uint32_t v_end, float *red_a,
                                         float *red_b, float *stats) {
     constexpr int EPV = Store<T>::EPV;
+    // half storage, long slices: unpack again in every pass instead of keeping K * 8 floats
+    // live; up to 5 vectors the unpacked copy fits the register file and is kept
+    constexpr bool kRepack = sizeof(T) == 2 && K > 5;
     const uint32_t tid = threadIdx.x;
     const uint32_t nt = blockDim.x;
     const u32x4 *xin = reinterpret_cast<const u32x4 *>(x) + (size_t)unit * p.vec_per_unit;
@@ -186,7 +189,7 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
     }
     const float slice_count = (float)((v_end - v_begin) * EPV);
     const float slice_mean = block_sum_rt(s, red_a) / slice_count;
-    if (sizeof(T) == 2) {
+    if (kRepack) {
 #pragma unroll
         for (int k = 0; k < K; k++) forget(raw[k]);
     }
@@ -207,7 +210,7 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
         q += qk;
     }
     const float slice_m2 = block_sum_rt(q, red_b);
-    if (sizeof(T) == 2) {
+    if (kRepack) {
 #pragma unroll
         for (int k = 0; k < K; k++) forget(raw[k]);
     }
@@ -325,6 +328,7 @@ __global__ __launch_bounds__(kGnMaxThreads) void gn_tokens_kernel(
     const T *__restrict__ x, T *__restrict__ y, const float *__restrict__ gamma,
     const float *__restrict__ beta, GnScratch scratch, GnTokParams q) {
     constexpr int EPV = Store<T>::EPV;
+    constexpr bool kRepack = sizeof(T) == 2 && K > 5;  // as in gn_body
     extern __shared__ u32x4 lds_vec[];
     __shared__ float red_a[kGnMaxThreads / kWave];
     __shared__ float red_b[kGnMaxThreads / kWave];
@@ -365,7 +369,7 @@ __global__ __launch_bounds__(kGnMaxThreads) void gn_tokens_kernel(
         s += (k * nt + tid < nvec) ? sk : 0.0f;
     }
     const float slice_mean = block_sum_rt(s, red_a) / (float)(nvec * EPV);
-    if (sizeof(T) == 2) {
+    if (kRepack) {
 #pragma unroll
         for (int k = 0; k < K; k++) forget(raw[k]);
     }
@@ -383,7 +387,7 @@ __global__ __launch_bounds__(kGnMaxThreads) void gn_tokens_kernel(
         m2 += (k * nt + tid < nvec) ? qk : 0.0f;
     }
     const float slice_m2 = block_sum_rt(m2, red_b);
-    if (sizeof(T) == 2) {
+    if (kRepack) {
 #pragma unroll
         for (int k = 0; k < K; k++) forget(raw[k]);
     }
@@ -569,6 +573,9 @@ int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma
         }
         while (units * want < 16 && want < kGnMaxSplit) want *= 2;  // very few units
         while (split < want && vec_per_unit >= (size_t)2 * split * 256) split *= 2;
+        // very long units (decoder-sized feature maps): keep a slice at 8 vectors per lane
+        // or fewer, which the 1024-lane register budget holds without spilling
+        while (split < kGnMaxSplit && (vec_per_unit + split - 1) / split > (size_t)kGnMaxThreads * 8) split *= 2;
     }
 
     GnParams p;

@@ -447,7 +447,10 @@ def test_groupnorm_many_units_and_register_limits(msd, orc, cuda):
     for shape, groups, half in [((300, 64, 4, 8), 32, True),     # 9600 units
                                 ((1, 32, 64, 64), 2, False),     # 65536-element float units
                                 ((2, 8, 128, 128), 1, False),    # 131072-element float units
-                                ((1, 16, 256, 256), 1, True)]:   # 1 Mi-element half unit: 64 slices
+                                ((1, 16, 256, 256), 1, True),    # 1 Mi-element half unit: 64 slices
+                                ((1, 128, 256, 256), 32, True),  # decoder-sized map, 262144-element units
+                                ((1, 128, 256, 256), 32, False),
+                                ((1, 4, 512, 512), 2, False)]:   # 524288-element float units
         x = orc.normal(shape, seed=sum(shape), sigma=1.7, mean=-0.3)
         xin = orc.round_to_half(x) if half else x
         g, b = _affine(orc, shape[1], 41)
