@@ -327,6 +327,7 @@ def load_nn_library(path=None):
     sig = {
         "msdnn_last_error": (cp, []),
         "msdnn_set_media_path": (None, [cp]),
+        "msdnn_set_debug_timing": (None, [it]),
         "msdnn_npy_load": (it, [cp, flp, sz, szp, szp]),
         "msdnn_npy_save": (it, [cp, flp, sz]),
         "msdnn_groupnorm_create": (vp, [vp, sz, sz, fl, cp, cp, sz, it]),

@@ -2,7 +2,9 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cstdio>
 #include <stdexcept>
+#include <string>
 
 #include "util.h"
 
@@ -93,6 +95,7 @@ int GroupNorm::run(const DeviceBuffer &input, const DeviceBuffer *chunk, DeviceB
     const size_t channelSize = input_size / num_channels;  // H*W (M/nn/GroupNorm.cpp:130)
     const float *w = static_cast<const float *>(bufferWeight.ptr());
     const float *b = static_cast<const float *>(bufferBias.ptr());
+    util::LaunchTimer timer(stream);
     const int rc = chunk ? msd_chunk_add_groupnorm(input.ptr(), chunk->ptr(), output.ptr(), w, b, batch,
                                                    num_channels, channelSize, num_groups, eps,
                                                    fuse_silu ? 1 : 0, (int)input.dtype(), stream)
@@ -100,6 +103,20 @@ int GroupNorm::run(const DeviceBuffer &input, const DeviceBuffer *chunk, DeviceB
                                          channelSize, num_groups, eps, fuse_silu ? 1 : 0,
                                          (int)input.dtype(), stream);
     if (rc != MSD_OK) return rc;
+    if (util::debugTiming()) {
+        // the reference's row (M/nn/GroupNorm.cpp:149-161), one kernel instead of three
+        static int count = 0;
+        if (count == 0)
+            fprintf(stderr, "try, component, index, input size, group size, num group, weight size, "
+                            "workgroup size, kernel, time(ms)\n");
+        const std::string message = "0, GroupNorm, " + std::to_string(count++) + ", " +
+                                    std::to_string(input_size) + ", " +
+                                    std::to_string(input_size / num_groups) + ", " +
+                                    std::to_string(num_groups) + ", " + std::to_string(weightSize) + ", " +
+                                    std::to_string(WORK_GROUP_SIZE);
+        timer.finish(message + (chunk ? ", chunk_add_group_norm" : ", group_norm") +
+                     (fuse_silu ? "_silu" : ""));
+    }
     if (event) return (int)hipEventRecord(event, stream);
     return MSD_OK;
 }

@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 
 #include <stdexcept>
+#include <string>
 
 #include "util.h"
 
@@ -33,6 +34,14 @@ void LayerNorm::init(const std::vector<float> &weight, const std::vector<float> 
     bufferBias = util::upload(bias, DType::F32, stream);
 }
 
+// The reference's timing row (M/nn/LayerNorm.cpp:144-154), one kernel instead of three.
+void LayerNorm::logTiming(util::LaunchTimer &timer, size_t input_size, const char *kernel) {
+    if (!util::debugTiming()) return;
+    static int count = 0;
+    timer.finish("2, LayerNorm, " + std::to_string(count++) + ", " + std::to_string(input_size) + ", " +
+                 std::to_string(weightSize) + ", " + kernel);
+}
+
 void LayerNorm::checkInput(size_t input_bytes, DType dtype) const {
     const size_t input_size = input_bytes / dtype_size(dtype);
     if (weightSize == 0 || input_size % weightSize != 0)
@@ -49,10 +58,12 @@ int LayerNorm::forward(const DeviceBuffer &input, DeviceBuffer &output, unsigned
         const hipError_t err = hipStreamWaitEvent(stream, event_wait_list[i], 0);
         if (err != hipSuccess) return (int)err;
     }
+    util::LaunchTimer timer(stream);
     const int rc = msd_layernorm(input.ptr(), output.ptr(), static_cast<const float *>(bufferWeight.ptr()),
                                  static_cast<const float *>(bufferBias.ptr()), input.count() / weightSize,
                                  weightSize, eps, (int)input.dtype(), stream);
     if (rc != MSD_OK) return rc;
+    logTiming(timer, input.count(), "layer_norm");
     if (event) return (int)hipEventRecord(event, stream);
     return MSD_OK;
 }
@@ -69,11 +80,13 @@ int LayerNorm::forwardAdd(const DeviceBuffer &a, const DeviceBuffer &b, DeviceBu
         const hipError_t err = hipStreamWaitEvent(stream, event_wait_list[i], 0);
         if (err != hipSuccess) return (int)err;
     }
+    util::LaunchTimer timer(stream);
     const int rc = msd_add_layernorm(a.ptr(), b.ptr(), sum.ptr(), output.ptr(),
                                      static_cast<const float *>(bufferWeight.ptr()),
                                      static_cast<const float *>(bufferBias.ptr()), a.count() / weightSize,
                                      weightSize, eps, (int)a.dtype(), stream);
     if (rc != MSD_OK) return rc;
+    logTiming(timer, a.count(), "add_layer_norm");
     if (event) return (int)hipEventRecord(event, stream);
     return MSD_OK;
 }

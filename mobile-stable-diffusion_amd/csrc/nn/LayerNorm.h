@@ -9,6 +9,7 @@
 #include <vector>
 
 #include "DeviceBuffer.h"
+#include "util.h"
 
 namespace msd {
 
@@ -39,6 +40,7 @@ public:
     void checkInput(size_t input_bytes, DType dtype) const;
 
 private:
+    void logTiming(util::LaunchTimer &timer, size_t input_size, const char *kernel);
     DeviceBuffer bufferWeight;
     DeviceBuffer bufferBias;
     size_t weightSize;

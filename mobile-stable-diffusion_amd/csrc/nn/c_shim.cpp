@@ -48,6 +48,9 @@ const char *msdnn_last_error(void) { return g_last_error.c_str(); }
 
 void msdnn_set_media_path(const char *dir) { util::setMediaPath(dir ? dir : ""); }
 
+// per-launch timing rows on stderr (the reference's DEBUG blocks); 0 switches them off
+void msdnn_set_debug_timing(int on) { util::setDebugTiming(on != 0); }
+
 // ---- npy (host only)
 int msdnn_npy_load(const char *name, float *out, size_t cap, size_t *num_vals, size_t *ndim) {
     return guarded([&] {

@@ -186,5 +186,40 @@ float printEventTime(const std::string &message, hipEvent_t start, hipEvent_t st
     return ms;
 }
 
+namespace {
+int g_debug_timing = -1;  // -1: not decided yet (environment), 0 off, 1 on
+}
+
+void setDebugTiming(bool on) { g_debug_timing = on ? 1 : 0; }
+
+bool debugTiming() {
+    if (g_debug_timing < 0) {
+        const char *env = getenv("MSD_DEBUG_TIMING");
+        g_debug_timing = (env && env[0] && env[0] != '0') ? 1 : 0;
+    }
+    return g_debug_timing == 1;
+}
+
+LaunchTimer::LaunchTimer(hipStream_t stream) : stream_(stream) {
+    if (!debugTiming()) return;
+    if (hipEventCreate(&start_) != hipSuccess || hipEventCreate(&stop_) != hipSuccess ||
+        hipEventRecord(start_, stream_) != hipSuccess) {
+        if (start_) (void)hipEventDestroy(start_);
+        if (stop_) (void)hipEventDestroy(stop_);
+        start_ = stop_ = nullptr;
+    }
+}
+
+LaunchTimer::~LaunchTimer() {
+    if (start_) (void)hipEventDestroy(start_);
+    if (stop_) (void)hipEventDestroy(stop_);
+}
+
+float LaunchTimer::finish(const std::string &message) {
+    if (!start_ || !stop_) return -1.0f;
+    if (hipEventRecord(stop_, stream_) != hipSuccess) return -1.0f;
+    return printEventTime(message, start_, stop_);
+}
+
 }  // namespace util
 }  // namespace msd

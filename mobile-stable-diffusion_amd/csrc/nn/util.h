@@ -49,5 +49,27 @@ TestResult testBuffer(const std::vector<float> &result, const char *filename);
 // util::printEventTime (M/util.cpp:203-215).  Returns the value (negative on error).
 float printEventTime(const std::string &message, hipEvent_t start, hipEvent_t stop);
 
+// Per-launch timing rows like the reference's `#define DEBUG 1` blocks
+// (M/nn/GroupNorm.cpp:147-162, M/nn/LayerNorm.cpp:144-154): switched on at run time by
+// setDebugTiming(true) or the MSD_DEBUG_TIMING=1 environment variable.  A LaunchTimer
+// brackets one launch with two events; finish() waits for it and prints
+// "<message>, <ms>" through printEventTime.  With timing off both calls do nothing.
+void setDebugTiming(bool on);
+bool debugTiming();
+class LaunchTimer {
+public:
+    explicit LaunchTimer(hipStream_t stream);
+    ~LaunchTimer();
+    LaunchTimer(const LaunchTimer &) = delete;
+    LaunchTimer &operator=(const LaunchTimer &) = delete;
+    // Returns the milliseconds (negative when timing is off or an event call failed).
+    float finish(const std::string &message);
+
+private:
+    hipStream_t stream_;
+    hipEvent_t start_ = nullptr;
+    hipEvent_t stop_ = nullptr;
+};
+
 }  // namespace util
 }  // namespace msd

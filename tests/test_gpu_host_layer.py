@@ -304,3 +304,35 @@ def test_ddim_sampler_object_walks_the_schedule_from_the_back(msd, nn, orc, cuda
     assert np.array_equal(xd.cpu().numpy(), x0)  # x_T untouched
     assert np.array_equal(out.cpu().numpy(), x)
     assert nn.msdnn_ddim_sample(None, _ptr(xd), n * 4, 0, 501, cb, None, _ptr(out)) < 0
+
+
+def test_debug_timing_rows_like_the_reference(msd, nn, orc, cuda, tmp_path, capfd):
+    """With timing on, each GroupNorm / LayerNorm forward prints the reference's CSV row
+    (M/nn/GroupNorm.cpp:147-162, M/nn/LayerNorm.cpp:144-154) with one kernel per layer."""
+    import torch
+    np.save(tmp_path / "w.npy", np.ones(320, dtype=np.float32))
+    np.save(tmp_path / "b.npy", np.zeros(320, dtype=np.float32))
+    g = nn.msdnn_groupnorm_create(None, 32, 320, 1e-5, b"w.npy", b"b.npy", 2, 1)
+    ln = nn.msdnn_layernorm_create(None, 320, b"w.npy", b"b.npy", 1e-5)
+    assert nn.msdnn_groupnorm_init(g) == 0 and nn.msdnn_layernorm_init(ln) == 0
+    x = torch.randn(2, 320, 16, 16, device=cuda)
+    y = torch.empty_like(x)
+    nbytes = x.numel() * 4
+    capfd.readouterr()
+    nn.msdnn_set_debug_timing(1)
+    try:
+        assert nn.msdnn_groupnorm_forward(g, _ptr(x), _ptr(y), nbytes, 0) == 0
+        assert nn.msdnn_layernorm_forward(ln, _ptr(x), _ptr(y), nbytes, 0) == 0
+    finally:
+        nn.msdnn_set_debug_timing(0)
+    err = capfd.readouterr().err
+    assert "try, component, index, input size, group size, num group, weight size, workgroup size, kernel" in err
+    gn_row = [l for l in err.splitlines() if l.startswith("0, GroupNorm, ")][-1].split(", ")
+    assert gn_row[3:8] == [str(320 * 256), str(10 * 256), "32", "320", "64"] and gn_row[8] == "group_norm_silu"
+    assert float(gn_row[9]) > 0.0
+    ln_row = [l for l in err.splitlines() if l.startswith("2, LayerNorm, ")][-1].split(", ")
+    assert ln_row[3:6] == [str(2 * 320 * 256), "320", "layer_norm"] and float(ln_row[6]) > 0.0
+    assert nn.msdnn_groupnorm_forward(g, _ptr(x), _ptr(y), nbytes, 0) == 0
+    assert "GroupNorm" not in capfd.readouterr().err  # off again
+    nn.msdnn_groupnorm_destroy(g)
+    nn.msdnn_layernorm_destroy(ln)
