@@ -164,6 +164,32 @@ class Step:
                     raise RuntimeError("%s failed: %d" % (kind, rc))
 
 
+class CopyStep:
+    """The same 133 launches with every kernel replaced by a plain 16-byte copy that moves the
+    same number of bytes (read + write) between buffers of its own: what the launch structure
+    and the tensor sizes alone cost on this machine."""
+
+    def __init__(self, msd, torch, dev):
+        import ctypes
+        self.lib = msd.load_library()
+        self.calls = []
+        self._keep = []
+        for kind, p in step_layers():
+            nb = layer_bytes(kind, p)
+            half = max(16, (nb // 2 + 15) // 16 * 16) if nb else 2 * BATCH * 1280  # bytes read = bytes written
+            src = torch.empty(half, dtype=torch.uint8, device=dev)
+            dst = torch.empty(half, dtype=torch.uint8, device=dev)
+            src.random_(0, 255)
+            self._keep += [src, dst]
+            self.calls.append((ctypes.c_void_p(src.data_ptr()), ctypes.c_void_p(dst.data_ptr()), half))
+
+    def run(self, stream_ptr):
+        for src, dst, nbytes in self.calls:
+            rc = self.lib.msd_copy(src, dst, nbytes, stream_ptr)
+            if rc != 0:
+                raise RuntimeError("copy failed: %d" % rc)
+
+
 def timed_replays(torch, fn, reps):
     """Wall time (s) of `reps` calls of fn, bracketed by device synchronisation."""
     torch.cuda.synchronize()
@@ -581,6 +607,18 @@ def main():
         ms_per_step = seconds * 1e3 / args.steps
         value = step.bytes / (seconds / args.steps) / 1e9
 
+        # the same launches as plain copies of the same bytes: the ceiling of this launch structure
+        copy_step = CopyStep(msd, torch, dev)
+
+        def eager_copy_step():
+            copy_step.run(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        run_copy = capture(torch, msd, stream, eager_copy_step) if args.mode == "graph" else eager_copy_step
+        for _ in range(max(3, args.warmup // 4)):
+            run_copy()
+        copy_reps = max(10, args.steps // 4)
+        copy_ms = timed_replays(torch, run_copy, copy_reps) * 1e3 / copy_reps
+        del copy_step
+
         # per-kernel-family timing inside the same step order (HIP events on the launch stream)
         families = {}
         for kind in ("gn_silu", "ln", "geglu"):
@@ -616,7 +654,8 @@ def main():
         "config": {"workload": "unet_step_norm_act: 45 GroupNorm(32)+SiLU, 48 LayerNorm, 16 GEGLU, 23 SiLU(emb), "
                                "1 timestep embedding at SD UNet shapes, batch 2, fp16 storage / fp32 arithmetic",
                    "bytes_per_step": step.bytes, "launches_per_step": len(step.launches), "launch_mode": args.mode,
-                   "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 1)},
+                   "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 1),
+                   "copy_step_ms": round(copy_ms, 4), "pct_of_copy_step_rate": round(100 * copy_ms / ms_per_step, 1)},
         "roofline": roofline,
         "kernel_families": families,
     }
