@@ -3,6 +3,7 @@
     libmsd_hip.so   HIP kernels + the C ABI declared in include/msd_hip.h
     libmsd_nn.so    C++ host layer objects (GroupNorm / LayerNorm / GEGLU / ...) on top of it
     cli/msd_compare golden-file comparison tool (host only)
+    cli/msd_layer_check  runs the layer objects against golden .npy files (needs a GPU)
 
 Run as a script (`python build.py`) or call build_all().
 """
@@ -27,6 +28,7 @@ DEVICE_FLAGS = [
 LIB_HIP = os.path.join(CSRC, "libmsd_hip.so")
 LIB_NN = os.path.join(CSRC, "libmsd_nn.so")
 CLI_COMPARE = os.path.join(CSRC, "cli", "msd_compare")
+CLI_LAYER_CHECK = os.path.join(CSRC, "cli", "msd_layer_check")
 
 
 def _run(cmd):
@@ -80,12 +82,24 @@ def build_cli():
     return CLI_COMPARE
 
 
+def build_layer_check():
+    """msd_layer_check: the layer objects against golden .npy files, from C++ alone."""
+    nn_dir = os.path.join(CSRC, "nn")
+    _run([os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-Wall", "-Wno-deprecated-declarations",
+          "-D__HIP_PLATFORM_AMD__", "-I", "/opt/rocm/include", "-I", os.path.join(REPO, "include"), "-I", nn_dir,
+          os.path.join(CSRC, "cli", "msd_layer_check.cpp"), "-o", CLI_LAYER_CHECK, "-L", CSRC, "-lmsd_nn",
+          "-lmsd_hip", "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,$ORIGIN/..", "-Wl,-rpath,/opt/rocm/lib"])
+    return CLI_LAYER_CHECK
+
+
 def build_all(verbose=True):
     built = [build_hip()]
     nn = build_nn()
     if nn:
         built.append(nn)
     built.append(build_cli())
+    if nn:
+        built.append(build_layer_check())
     if verbose:
         for b in built:
             print("built", b)

@@ -336,3 +336,63 @@ def test_debug_timing_rows_like_the_reference(msd, nn, orc, cuda, tmp_path, capf
     assert "GroupNorm" not in capfd.readouterr().err  # off again
     nn.msdnn_groupnorm_destroy(g)
     nn.msdnn_layernorm_destroy(ln)
+
+
+def test_layer_objects_from_cpp_against_golden_files(orc, cuda, tmp_path):
+    """msd_layer_check: a C++ program that uses only the public layer headers, driven like the
+    reference's in-source checks (weights and goldens as .npy under the media path)."""
+    import os
+    import subprocess
+    repo = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    tool = os.path.join(repo, "mobile-stable-diffusion_amd", "csrc", "cli", "msd_layer_check")
+    assert os.path.exists(tool), "msd_layer_check is not built: run __graft_entry__.build()"
+    rnd = orc.round_to_half
+    lines = []
+
+    def save(name, a):
+        np.save(tmp_path / name, np.ascontiguousarray(a, dtype=np.float32))
+        return name
+
+    # ResBlock in-norm + SiLU, fp32 and fp16 storage, batch 2
+    w = orc.normal((320,), seed=601, mean=1.0, sigma=0.1)
+    b = orc.normal((320,), seed=602, sigma=0.1)
+    x = orc.normal((2, 320, 32, 32), seed=603, sigma=2.0)
+    save("gn_w.npy", w), save("gn_b.npy", b), save("gn_x.npy", x), save("gn_x16.npy", rnd(x))
+    save("gn_golden.npy", orc.groupnorm(x, w, b, 32, 1e-5, silu=True))
+    save("gn_golden16.npy", rnd(orc.groupnorm(rnd(x), w, b, 32, 1e-5, silu=True)))
+    lines.append("groupnorm 320 32 1e-5 2 1 f32 gn_w.npy gn_b.npy gn_x.npy gn_golden.npy")
+    lines.append("groupnorm 320 32 1e-5 2 1 f16 gn_w.npy gn_b.npy gn_x16.npy gn_golden16.npy")
+    # transformer LayerNorm and GEGLU
+    xl = orc.normal((2 * 1024, 640), seed=604)
+    wl = orc.normal((640,), seed=605, mean=1.0, sigma=0.1)
+    bl = orc.normal((640,), seed=606, sigma=0.1)
+    save("ln_w.npy", wl), save("ln_b.npy", bl), save("ln_x.npy", xl)
+    save("ln_golden.npy", orc.layernorm(xl, wl, bl, 1e-5))
+    lines.append("layernorm 640 1e-5 f32 ln_w.npy ln_b.npy ln_x.npy ln_golden.npy")
+    proj = rnd(orc.normal((512, 2 * 1280), seed=607, sigma=1.5))
+    save("geglu_x.npy", proj), save("geglu_golden.npy", rnd(orc.geglu(proj)))
+    lines.append("geglu 320 1280 f16 geglu_x.npy geglu_golden.npy")
+    # time embedding Linear with SiLU behind it, ResBlock projection with SiLU in front, no bias case
+    wt = orc.normal((1280, 320), seed=608, sigma=320 ** -0.5)
+    bt = orc.normal((1280,), seed=609, sigma=0.1)
+    te = np.stack([orc.timestep_embedding(t) for t in (981, 1)])
+    save("te_w.npy", wt), save("te_b.npy", bt), save("te_x.npy", te)
+    save("te_golden.npy", orc.silu(orc.linear(te, wt, bt)))
+    lines.append("linear 320 1280 0 1 f32 te_w.npy te_b.npy te_x.npy te_golden.npy")
+    save("te_golden_nobias.npy", orc.linear(orc.silu(te), wt, None))
+    lines.append("linear 320 1280 1 0 f32 te_w.npy - te_x.npy te_golden_nobias.npy")
+    # cross-attention softmax, in place
+    qk = orc.normal((8 * 256, 77), seed=610, sigma=2.0)
+    save("sm_x.npy", qk), save("sm_golden.npy", orc.softmax(qk))
+    lines.append("softmax 77 0 f32 sm_x.npy sm_golden.npy")
+    # a golden that must fail (wrong SiLU flag) and a missing weight file: reported, not fatal
+    lines.append("groupnorm 320 32 1e-5 2 0 f32 gn_w.npy gn_b.npy gn_x.npy gn_golden.npy")
+    lines.append("layernorm 640 1e-5 f32 nope.npy ln_b.npy ln_x.npy ln_golden.npy")
+    (tmp_path / "manifest.txt").write_text("# cases\n" + "\n".join(lines) + "\n")
+    p = subprocess.run([tool, str(tmp_path), str(tmp_path / "manifest.txt")], stdout=subprocess.PIPE,
+                       stderr=subprocess.PIPE, text=True, timeout=100)
+    out = p.stdout.splitlines()
+    verdicts = [l.split()[0] for l in out if l.startswith(("PASS", "FAIL"))]
+    assert verdicts == ["PASS"] * 7 + ["FAIL", "FAIL"], p.stdout + p.stderr
+    assert p.returncode == 2 and out[-1] == "7 of 9 cases passed"
+    assert "max diff:" in p.stderr and "Unable to open file" in p.stderr
