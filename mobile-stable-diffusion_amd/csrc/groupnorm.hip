@@ -321,6 +321,7 @@ struct GnTokParams {
     uint32_t hw;          // positions per sample
     uint32_t channels;
     uint32_t pitch;       // LDS elements between channels: positions per slice + 16 bytes
+    FastDiv combos;       // batch * split: (sample, slice) pairs, the fastest part of the block id
 };
 
 template <typename T, int K>
@@ -336,8 +337,15 @@ __global__ __launch_bounds__(kGnMaxThreads) void gn_tokens_kernel(
     const GnParams &p = q.base;
     const uint32_t tid = threadIdx.x;
     const uint32_t nt = blockDim.x;
-    const uint32_t unit = blockIdx.x >> p.split_shift;
-    const uint32_t slice = blockIdx.x & (p.split - 1);
+    // block id = group * (batch * split) + sample * split + slice: the workgroups that write
+    // pieces of the same output lines (all groups of one sample and position range) have ids
+    // that differ by multiples of batch * split, so with workgroups dealt round-robin to the
+    // 8 XCDs they meet in one L2 when that product is a multiple of 8 (batch 2 x 4 slices);
+    // the slices of a unit stay adjacent
+    const uint32_t group = fast_div(blockIdx.x, q.combos);
+    const uint32_t combo = blockIdx.x - group * q.combos.d;
+    const uint32_t unit = (combo >> p.split_shift) * p.groups + group;
+    const uint32_t slice = combo & (p.split - 1);
     const uint32_t nvec = p.vec_per_slice;
     const uint32_t pvs = q.pos_vecs.d;
     const u32x4 *xin = reinterpret_cast<const u32x4 *>(x) + (size_t)unit * p.vec_per_unit;
@@ -663,8 +671,10 @@ int gn_tokens_dispatch(const void *xv, void *yv, const float *gamma, const float
     if (!vector_ok) return generic();
     const size_t hw_vec = hw / EPV;
     // slices cut the positions: the split must divide them, fit the registers and the LDS
+    // (cut earlier than gn_dispatch does: with batch * split = 8 the writers of an output line
+    // share an XCD, which is worth more than the exchange costs from 16 Ki elements on)
     uint32_t want = 1;
-    if (unit_size > 24576) {
+    if (unit_size > 16384) {
         want = 4;
         if (units * 4 < 192 && unit_size >= 65536) want = 8;
     }
@@ -697,6 +707,7 @@ int gn_tokens_dispatch(const void *xv, void *yv, const float *gamma, const float
     q.hw = (uint32_t)hw;
     q.channels = (uint32_t)channels;
     q.pitch = (uint32_t)(pvs * EPV + 16 / sizeof(T));
+    q.combos = make_fast_div((uint32_t)(batch * split));
     const size_t lds_bytes = cpg * q.pitch * sizeof(T);
     const GnPlan pl = plan_slice((uint32_t)nvec, split, 0, kMaxK);
     if (pl.k == 0) return generic();
