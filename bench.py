@@ -8,7 +8,7 @@ each layer on its own HBM-resident buffers, launched back to back on one stream.
 `value` = algorithmic bytes of one step / time per step.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode graph|eager]
-                    [--no-cpu] [--no-shapes] [--tables shapes,fusions,neighbours]
+                    [--no-cpu] [--no-shapes] [--tables shapes,fusions,neighbours,large_batch]
 
 Prints ONE JSON line (see the keys below).  The CPU oracle is used only for the
 `cpu_baseline` leg.
@@ -490,6 +490,65 @@ def neighbour_table(torch, msd, dev, stream):
     return rows
 
 
+def large_batch_table(torch, msd, dev, stream):
+    """The same kernels on tensors 16 times larger than the UNet step's (batch 32), where the
+    1.6 us launch floor no longer matters: what each kernel sustains against a plain copy."""
+    import ctypes
+    vp = ctypes.c_void_p
+    lib = msd.load_library()
+    F16 = msd.DTYPE_F16
+    B = 32
+    rows = []
+
+    def sp():
+        return vp(torch.cuda.current_stream().cuda_stream)
+
+    def measure(fn, launches):
+        replay = capture(torch, msd, stream, fn)
+        with torch.cuda.stream(stream):
+            replay()
+            reps = max(3, 60 // launches)
+            return event_time_ms(torch, replay, reps) * 1e3 / (reps * launches)
+
+    cases = [("groupnorm_silu", {"batch": B, "c": 320, "hw": 4096}, B * 320 * 4096, B * 320 * 4096),
+             ("layernorm", {"rows": B * 4096, "dim": 320}, B * 4096 * 320, B * 4096 * 320),
+             ("geglu", {"rows": B * 4096, "inner": 1280}, B * 4096 * 2560, B * 4096 * 1280)]
+    for kind, p, n_in, n_out in cases:
+        copies = 3
+        xs = [torch.randn(n_in, device=dev).half() for _ in range(copies)]
+        ys = [torch.empty(n_out, device=dev, dtype=torch.float16) for _ in range(copies)]
+        d = p.get("c", p.get("dim", 1))
+        ga, be = torch.ones(d, device=dev), torch.zeros(d, device=dev)
+
+        def body():
+            for x, y in zip(xs, ys):
+                if kind == "groupnorm_silu":
+                    rc = lib.msd_groupnorm(vp(x.data_ptr()), vp(y.data_ptr()), vp(ga.data_ptr()), vp(be.data_ptr()),
+                                           B, p["c"], p["hw"], 32, 1e-5, 1, F16, sp())
+                elif kind == "layernorm":
+                    rc = lib.msd_layernorm(vp(x.data_ptr()), vp(y.data_ptr()), vp(ga.data_ptr()), vp(be.data_ptr()),
+                                           p["rows"], p["dim"], 1e-5, F16, sp())
+                else:
+                    rc = lib.msd_geglu(vp(x.data_ptr()), vp(y.data_ptr()), p["rows"], p["inner"], F16, sp())
+                assert rc == 0
+
+        def copy_body():  # the same total bytes: read half, write half
+            for x, y in zip(xs, ys):
+                assert lib.msd_copy(vp(x.data_ptr()), vp(y.data_ptr()), 2 * n_out, sp()) == 0
+        nbytes = 2 * (n_in + n_out)
+        us = measure(body, copies)
+        row = {"kernel": kind, "shape": p, "dtype": "f16", "bytes": nbytes, "us": round(us, 2),
+               "GBps": round(nbytes / us / 1e3, 1), "pct_hbm_peak": round(100 * nbytes / us / 1e3 / HBM_PEAK_GBS, 1)}
+        if n_in == n_out:
+            cus = measure(copy_body, copies)
+            row["copy_us"] = round(cus, 2)
+            row["pct_of_copy_rate"] = round(100 * cus / us, 1)
+        rows.append(row)
+        del xs, ys
+        torch.cuda.empty_cache()
+    return rows
+
+
 def cpu_baseline(total_bytes, budget_s=24.0):
     """The reference path as host loops (the CPU oracle, fp32, unfused passes exactly as the
     reference enqueues them) over the layers of one full step, timed on this host's cores.
@@ -556,7 +615,7 @@ def main():
     ap.add_argument("--mode", choices=["graph", "eager"], default="graph")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-kernel tables")
-    ap.add_argument("--tables", default="shapes,fusions,neighbours",
+    ap.add_argument("--tables", default="shapes,fusions,neighbours,large_batch",
                     help="comma list of the per-kernel tables to measure")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="for rocprofv3 --pmc runs: one 64 MiB device copy (known traffic) then three "
@@ -664,6 +723,8 @@ def main():
         out["shapes"] = shape_table(torch, msd, dev, stream)
     if "fusions" in tables:
         out["fusions"] = fusion_table(torch, msd, dev, stream)
+    if "large_batch" in tables:
+        out["large_batch"] = large_batch_table(torch, msd, dev, stream)
     if "neighbours" in tables:
         out["neighbours"] = neighbour_table(torch, msd, dev, stream)
     if not args.no_cpu:

@@ -442,6 +442,16 @@ def test_groupnorm_two_streams_have_private_scratch(msd, orc, cuda):
     assert lib.msd_status(ctypes.c_void_p(s2.cuda_stream)) == 0
 
 
+@pytest.mark.parametrize("batch,channels,hw", [(8, 320, 4096), (4, 640, 4096), (8, 960, 1024), (5, 320, 4096)])
+def test_groupnorm_larger_batches_pick_other_splits(msd, orc, cuda, batch, channels, hw):
+    # 128 / 256 units: the launch plan cuts units in two or not at all instead of in four
+    x = orc.normal((batch, channels, hw), seed=batch * 1000 + channels, sigma=1.5, mean=0.2)
+    g, b = _affine(orc, channels, 77)
+    _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half=True)
+    _run_groupnorm(msd, orc, cuda, x[:, :, : hw // 4], g, b, 32, 1e-5, True, half=False)
+    assert msd.status() == 0
+
+
 def test_groupnorm_many_units_and_register_limits(msd, orc, cuda):
     # more units than scratch slots (never split), and float units that need a split to fit
     for shape, groups, half in [((300, 64, 4, 8), 32, True),     # 9600 units
