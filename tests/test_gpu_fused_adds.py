@@ -109,7 +109,8 @@ def test_add_layernorm_equals_two_launches(msd, orc, cuda, rows, dim, half):
                                                 ((2, 1280, 16, 16), 32, 0), ((2, 1280, 8, 8), 32, 0),
                                                 ((1, 320, 64, 64), 32, 8), ((2, 640, 32, 32), 32, 2),
                                                 ((1, 96, 24, 24), 32, 0), ((3, 64, 5, 7), 8, 0),
-                                                ((1, 33, 4, 4), 33, 0), ((1, 8, 128, 128), 1, 0)])
+                                                ((1, 33, 4, 4), 33, 0), ((1, 8, 128, 128), 1, 0),
+                                                ((8, 320, 32, 32), 32, 0), ((4, 640, 32, 32), 32, 0)])
 def test_groupnorm_tokens_equals_norm_then_permute(msd, orc, cuda, shape, groups, split, half):
     """SpatialTransformer's GroupNorm(eps 1e-6, no SiLU) + permute (0, 2, 1) in one launch
     (M/nn/SpatialTransformer.cpp:127-139)."""
