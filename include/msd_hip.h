@@ -40,7 +40,10 @@ const char *msd_error_string(int code);
  * statistics that workgroups sharing one GroupNorm group exchange) ahead of
  * time.  Optional: msd_groupnorm creates it on first use; call this first
  * when the first msd_groupnorm on a stream would otherwise happen under
- * stream capture.  No reference counterpart (the reference allocates two
+ * stream capture.  A graph captured on a stream keeps using that stream's
+ * scratch: GroupNorm launches that share scratch must not run concurrently
+ * (do not replay such a graph on a second stream while the first is busy with
+ * GroupNorms).  No reference counterpart (the reference allocates two
  * temporaries per forward, M/nn/GroupNorm.cpp:95-103).
  */
 int msd_init(void *stream);
