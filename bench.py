@@ -27,7 +27,7 @@ if REPO not in sys.path:
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # measured HBM bytes per geglu_kernel<__half> launch, averaged over the 16 launches of a step
 # (rocprofv3 counters; algorithmic figure is 34652160)
-GEGLU_TRAFFIC_BYTES_PER_LAUNCH = 34683534
+GEGLU_TRAFFIC_BYTES_PER_LAUNCH = 34683383
 
 
 # ----------------------------------------------------------------------------
