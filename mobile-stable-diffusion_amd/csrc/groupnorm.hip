@@ -114,6 +114,77 @@ __device__ __forceinline__ void gn_exchange(const GnScratch &scratch, const GnPa
     __syncthreads();
 }
 
+// Mean and M2 = sum (x - mean)^2 of the workgroup's slice, held as K packed vectors per lane
+// (vector k of lane t is element k * blockDim.x + t of the slice; the first n_valid count).
+// Each wavefront reduces its own part in two passes with DPP only, the parts meet once in LDS
+// (one barrier), and every wavefront merges them with Chan's formula, lane l taking
+// wavefront l's entry.  FULL: every lane owns exactly K valid vectors.
+template <typename T, int K, bool FULL>
+__device__ __forceinline__ void gn_slice_stats(u32x4 (&raw)[K], uint32_t n_valid, float *red_a,
+                                               float *red_b, float *red_c, float &slice_mean,
+                                               float &slice_m2) {
+    constexpr int EPV = Store<T>::EPV;
+    // half storage, long slices: unpack again in every pass instead of keeping K * 8 floats
+    // live; up to 8 vectors the unpacked copy fits the register file and is kept
+    constexpr bool kRepack = sizeof(T) == 2 && K > 8;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t nt = blockDim.x;
+    const uint32_t lane = tid & (kWave - 1);
+    float s = 0.0f, cnt = 0.0f;
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        float f[EPV];
+        Store<T>::unpack(raw[k], f);
+        float sk = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EPV; e++) sk += f[e];
+        if (!FULL) {
+            const bool have = k * nt + tid < n_valid;
+            sk = have ? sk : 0.0f;
+            cnt += have ? (float)EPV : 0.0f;
+        }
+        s += sk;
+    }
+    const float wave_cnt = FULL ? (float)(kWave * K * EPV) : wave_sum(cnt);
+    const float wave_mean = wave_sum(s) / fmaxf(wave_cnt, 1.0f);
+    if (kRepack) {
+#pragma unroll
+        for (int k = 0; k < K; k++) forget(raw[k]);
+    }
+    float q = 0.0f;
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        float f[EPV];
+        Store<T>::unpack(raw[k], f);
+        float qk = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EPV; e++) {
+            const float d = f[e] - wave_mean;
+            qk = fmaf(d, d, qk);
+        }
+        if (!FULL) qk = (k * nt + tid < n_valid) ? qk : 0.0f;
+        q += qk;
+    }
+    const float wave_m2 = wave_sum(q);
+    if (kRepack) {
+#pragma unroll
+        for (int k = 0; k < K; k++) forget(raw[k]);
+    }
+    if (lane == 0) {
+        red_a[tid / kWave] = wave_mean;
+        red_b[tid / kWave] = wave_m2;
+        red_c[tid / kWave] = wave_cnt;
+    }
+    __syncthreads();
+    const bool entry = lane < nt / kWave;
+    const float m_l = entry ? red_a[lane] : 0.0f;
+    const float q_l = entry ? red_b[lane] : 0.0f;
+    const float n_l = entry ? red_c[lane] : 0.0f;
+    slice_mean = wave_sum(m_l * n_l) / (float)(n_valid * EPV);
+    const float dm = m_l - slice_mean;
+    slice_m2 = wave_sum(fmaf(n_l * dm, dm, q_l));
+}
+
 // FULL: every lane owns exactly K vectors (no masking anywhere).
 template <typename T, int K, bool SILU, bool FULL>
 __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
@@ -121,11 +192,8 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
                                         const float *__restrict__ beta, const GnScratch &scratch,
                                         const GnParams &p, uint32_t unit, uint32_t slice,
                                         uint32_t v_begin, uint32_t v_end, float *red_a,
-                                        float *red_b, float *stats) {
+                                        float *red_b, float *red_c, float *stats) {
     constexpr int EPV = Store<T>::EPV;
-    // half storage, long slices: unpack again in every pass instead of keeping K * 8 floats
-    // live; up to 5 vectors the unpacked copy fits the register file and is kept
-    constexpr bool kRepack = sizeof(T) == 2 && K > 5;
     const uint32_t tid = threadIdx.x;
     const uint32_t nt = blockDim.x;
     const u32x4 *xin = reinterpret_cast<const u32x4 *>(x) + (size_t)unit * p.vec_per_unit;
@@ -175,45 +243,8 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
         }
     }
 
-    // ---- slice mean
-    float s = 0.0f;
-#pragma unroll
-    for (int k = 0; k < K; k++) {
-        float f[EPV];
-        Store<T>::unpack(raw[k], f);
-        float sk = 0.0f;
-#pragma unroll
-        for (int e = 0; e < EPV; e++) sk += f[e];
-        if (!FULL) sk = (v_begin + k * nt + tid < v_end) ? sk : 0.0f;
-        s += sk;
-    }
-    const float slice_count = (float)((v_end - v_begin) * EPV);
-    const float slice_mean = block_sum_rt(s, red_a) / slice_count;
-    if (kRepack) {
-#pragma unroll
-        for (int k = 0; k < K; k++) forget(raw[k]);
-    }
-
-    // ---- slice M2
-    float q = 0.0f;
-#pragma unroll
-    for (int k = 0; k < K; k++) {
-        float f[EPV];
-        Store<T>::unpack(raw[k], f);
-        float qk = 0.0f;
-#pragma unroll
-        for (int e = 0; e < EPV; e++) {
-            const float d = f[e] - slice_mean;
-            qk = fmaf(d, d, qk);
-        }
-        if (!FULL) qk = (v_begin + k * nt + tid < v_end) ? qk : 0.0f;
-        q += qk;
-    }
-    const float slice_m2 = block_sum_rt(q, red_b);
-    if (kRepack) {
-#pragma unroll
-        for (int k = 0; k < K; k++) forget(raw[k]);
-    }
+    float slice_mean, slice_m2;
+    gn_slice_stats<T, K, FULL>(raw, v_end - v_begin, red_a, red_b, red_c, slice_mean, slice_m2);
 
     float mean, rstd;
     if (p.split == 1) {
@@ -256,6 +287,7 @@ __global__ __launch_bounds__(kGnMaxThreads) void gn_slice_kernel(
     const float *__restrict__ beta, GnScratch scratch, GnParams p) {
     __shared__ float red_a[kGnMaxThreads / kWave];
     __shared__ float red_b[kGnMaxThreads / kWave];
+    __shared__ float red_c[kGnMaxThreads / kWave];
     __shared__ float stats[2];
     const uint32_t unit = blockIdx.x >> p.split_shift;
     const uint32_t slice = blockIdx.x & (p.split - 1);
@@ -263,10 +295,10 @@ __global__ __launch_bounds__(kGnMaxThreads) void gn_slice_kernel(
     const uint32_t v_end = min(p.vec_per_unit, v_begin + p.vec_per_slice);
     if (v_end - v_begin == K * blockDim.x)  // uniform over the workgroup
         gn_body<T, K, SILU, true>(x, chunk, y, gamma, beta, scratch, p, unit, slice, v_begin, v_end,
-                                  red_a, red_b, stats);
+                                  red_a, red_b, red_c, stats);
     else
         gn_body<T, K, SILU, false>(x, chunk, y, gamma, beta, scratch, p, unit, slice, v_begin, v_end,
-                                   red_a, red_b, stats);
+                                   red_a, red_b, red_c, stats);
 }
 
 // Any shape or alignment: one workgroup per unit, three passes over global memory with
@@ -329,10 +361,10 @@ __global__ __launch_bounds__(kGnMaxThreads) void gn_tokens_kernel(
     const T *__restrict__ x, T *__restrict__ y, const float *__restrict__ gamma,
     const float *__restrict__ beta, GnScratch scratch, GnTokParams q) {
     constexpr int EPV = Store<T>::EPV;
-    constexpr bool kRepack = sizeof(T) == 2 && K > 5;  // as in gn_body
     extern __shared__ u32x4 lds_vec[];
     __shared__ float red_a[kGnMaxThreads / kWave];
     __shared__ float red_b[kGnMaxThreads / kWave];
+    __shared__ float red_c[kGnMaxThreads / kWave];
     __shared__ float stats[2];
     const GnParams &p = q.base;
     const uint32_t tid = threadIdx.x;
@@ -366,39 +398,8 @@ __global__ __launch_bounds__(kGnMaxThreads) void gn_tokens_kernel(
     }
     const uint32_t ch0 = (unit % p.groups) * p.ch_per_group;
 
-    float s = 0.0f;
-#pragma unroll
-    for (int k = 0; k < K; k++) {
-        float f[EPV];
-        Store<T>::unpack(raw[k], f);
-        float sk = 0.0f;
-#pragma unroll
-        for (int e = 0; e < EPV; e++) sk += f[e];
-        s += (k * nt + tid < nvec) ? sk : 0.0f;
-    }
-    const float slice_mean = block_sum_rt(s, red_a) / (float)(nvec * EPV);
-    if (kRepack) {
-#pragma unroll
-        for (int k = 0; k < K; k++) forget(raw[k]);
-    }
-    float m2 = 0.0f;
-#pragma unroll
-    for (int k = 0; k < K; k++) {
-        float f[EPV];
-        Store<T>::unpack(raw[k], f);
-        float qk = 0.0f;
-#pragma unroll
-        for (int e = 0; e < EPV; e++) {
-            const float d = f[e] - slice_mean;
-            qk = fmaf(d, d, qk);
-        }
-        m2 += (k * nt + tid < nvec) ? qk : 0.0f;
-    }
-    const float slice_m2 = block_sum_rt(m2, red_b);
-    if (kRepack) {
-#pragma unroll
-        for (int k = 0; k < K; k++) forget(raw[k]);
-    }
+    float slice_mean, slice_m2;
+    gn_slice_stats<T, K, false>(raw, nvec, red_a, red_b, red_c, slice_mean, slice_m2);
 
     float mean, rstd;
     if (p.split == 1) {
