@@ -504,7 +504,7 @@ GnPlan plan_slice(uint32_t vecs, uint32_t split, uint32_t force_threads, uint32_
     GnPlan pl{split, 0, 0};
     if (force_threads)
         pl.threads = force_threads;
-    else if (vecs > 512u * 5u)
+    else if (vecs > 512u * 5u || (split > 1 && vecs >= 960))  // slices of a cut unit: 2 - 3 % faster
         pl.threads = kGnMaxThreads;
     else if (vecs >= 256)
         pl.threads = 512;
