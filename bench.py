@@ -200,17 +200,23 @@ def timed_replays(torch, fn, reps):
     return time.perf_counter() - t0
 
 
-def event_time_ms(torch, fn, reps):
-    """Elapsed GPU time (ms) of `reps` calls of fn between two HIP events recorded on
-    the stream the kernels are launched on (torch's current stream)."""
-    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    a.record()
-    for _ in range(reps):
-        fn()
-    b.record()
-    b.synchronize()
-    return a.elapsed_time(b)
+def event_time_ms(torch, fn, reps, batches=5):
+    """Elapsed GPU time (ms) of `reps` calls of fn between two HIP events recorded on the
+    stream the kernels are launched on (torch's current stream): the median of `batches`
+    such measurements, each of reps / batches calls scaled back to `reps`."""
+    per = max(1, reps // batches)
+    times = []
+    for _ in range(batches):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        a.record()
+        for _ in range(per):
+            fn()
+        b.record()
+        b.synchronize()
+        times.append(a.elapsed_time(b) / per)
+    times.sort()
+    return times[len(times) // 2] * reps
 
 
 def capture(torch, msd, stream, body):
@@ -287,7 +293,8 @@ def shape_table(torch, msd, dev, stream):
                     continue
                 replay = capture(torch, msd, stream, fn)
                 with torch.cuda.stream(stream):
-                    replay()
+                    for _ in range(20 // copies + 1):  # at least 20 warm-up launches
+                        replay()
                     us[name] = event_time_ms(torch, replay, reps) * 1e3 / (reps * copies)
             gbs = nbytes / us["kernel"] / 1e3
             row = {"kernel": kind, "shape": p, "dtype": "f16" if elt == 2 else "f32",
