@@ -556,6 +556,106 @@ def large_batch_table(torch, msd, dev, stream):
     return rows
 
 
+def step_with_adds(torch, msd, dev, stream):
+    """One UNet step of the path including the additions the reference runs right before its
+    norms (the embedding add before each ResBlock out-norm, the residual add before LayerNorm 2
+    and 3 of each transformer block): as separate launches in the reference's order, and
+    folded into the norm kernels.  Same buffers, graph-replayed."""
+    import ctypes
+    vp = ctypes.c_void_p
+    lib = msd.load_library()
+    F16 = msd.DTYPE_F16
+    g = torch.Generator(device=dev).manual_seed(77)
+    keep = []
+
+    def randn(*shape, dtype=torch.float16):
+        t = torch.randn(*shape, device=dev, dtype=torch.float32, generator=g).to(dtype)
+        keep.append(t)
+        return t
+
+    affine = {}
+
+    def gb(c):
+        if c not in affine:
+            affine[c] = (1.0 + 0.1 * randn(c, dtype=torch.float32), 0.1 * randn(c, dtype=torch.float32))
+        return affine[c]
+
+    separate, fused = [], []  # lists of (fn, args)
+    out_norm, ln_count = False, 0
+    for kind, p in step_layers():
+        if kind == "temb":
+            t = torch.randint(0, 1000, (BATCH,), device=dev, dtype=torch.int64, generator=g)
+            out = torch.empty((BATCH, p["dim"]), device=dev, dtype=torch.float16)
+            keep += [t, out]
+            call = (lib.msd_timestep_embedding, (vp(t.data_ptr()), vp(out.data_ptr()), BATCH, p["dim"], 10000.0, F16))
+            separate.append(call), fused.append(call)
+        elif kind == "silu":
+            x = randn(p["n"])
+            call = (lib.msd_silu, (vp(x.data_ptr()), vp(x.data_ptr()), p["n"], F16))
+            separate.append(call), fused.append(call)
+            out_norm = True  # the next GroupNorm is the ResBlock's out-norm (after the embedding add)
+        elif kind == "gn_silu":
+            c, hw = p["c"], p["hw"]
+            x = randn(BATCH, c, hw) * 2.0
+            keep.append(x)
+            y = x if p["inplace"] else torch.empty_like(x)
+            keep.append(y)
+            ga, be = gb(c)
+            xp, yp = vp(x.data_ptr()), vp(y.data_ptr())
+            gp, bp = vp(ga.data_ptr()), vp(be.data_ptr())
+            if out_norm and p["inplace"]:
+                emb = randn(BATCH * c)
+                ep = vp(emb.data_ptr())
+                separate.append((lib.msd_chunkwise_add, (xp, ep, xp, BATCH * c * hw, hw, F16)))
+                separate.append((lib.msd_groupnorm, (xp, yp, gp, bp, BATCH, c, hw, 32, 1e-5, 1, F16)))
+                fused.append((lib.msd_chunk_add_groupnorm, (xp, ep, yp, gp, bp, BATCH, c, hw, 32, 1e-5, 1, F16)))
+                out_norm = False
+            else:
+                call = (lib.msd_groupnorm, (xp, yp, gp, bp, BATCH, c, hw, 32, 1e-5, 1, F16))
+                separate.append(call), fused.append(call)
+        elif kind == "ln":
+            rows, dim = p["rows"], p["dim"]
+            x, y = randn(rows, dim), torch.empty((rows, dim), device=dev, dtype=torch.float16)
+            keep.append(y)
+            ga, be = gb(dim)
+            xp, yp, gp, bp = vp(x.data_ptr()), vp(y.data_ptr()), vp(ga.data_ptr()), vp(be.data_ptr())
+            if ln_count % 3 == 0:  # LayerNorm 1 of a block has no add in front
+                call = (lib.msd_layernorm, (xp, yp, gp, bp, rows, dim, 1e-5, F16))
+                separate.append(call), fused.append(call)
+            else:
+                res = randn(rows, dim)
+                rp = vp(res.data_ptr())
+                separate.append((lib.msd_elemwise_add, (xp, rp, xp, rows * dim, F16)))
+                separate.append((lib.msd_layernorm, (xp, yp, gp, bp, rows, dim, 1e-5, F16)))
+                fused.append((lib.msd_add_layernorm, (xp, rp, xp, yp, gp, bp, rows, dim, 1e-5, F16)))
+            ln_count += 1
+        else:
+            rows, inner = p["rows"], p["inner"]
+            x = randn(rows, 2 * inner)
+            y = torch.empty((rows, inner), device=dev, dtype=torch.float16)
+            keep.append(y)
+            call = (lib.msd_geglu, (vp(x.data_ptr()), vp(y.data_ptr()), rows, inner, F16))
+            separate.append(call), fused.append(call)
+
+    def runner(calls):
+        def run():
+            sp = vp(torch.cuda.current_stream().cuda_stream)
+            for fn, args in calls:
+                assert fn(*args, sp) == 0
+        return run
+
+    out = {}
+    for name, calls in (("separate", separate), ("fused", fused)):
+        replay = capture(torch, msd, stream, runner(calls))
+        with torch.cuda.stream(stream):
+            for _ in range(5):
+                replay()
+            out[name] = event_time_ms(torch, replay, 50) / 50
+    return {"launches_separate": len(separate), "launches_fused": len(fused),
+            "ms_separate": round(out["separate"], 4), "ms_fused": round(out["fused"], 4),
+            "speedup": round(out["separate"] / out["fused"], 3)}
+
+
 def cpu_baseline(total_bytes, budget_s=24.0):
     """The reference path as host loops (the CPU oracle, fp32, unfused passes exactly as the
     reference enqueues them) over the layers of one full step, timed on this host's cores.
@@ -730,6 +830,8 @@ def main():
         out["shapes"] = shape_table(torch, msd, dev, stream)
     if "fusions" in tables:
         out["fusions"] = fusion_table(torch, msd, dev, stream)
+    if "fusions" in tables:
+        out["step_with_adds"] = step_with_adds(torch, msd, dev, stream)
     if "large_batch" in tables:
         out["large_batch"] = large_batch_table(torch, msd, dev, stream)
     if "neighbours" in tables:
