@@ -48,7 +48,9 @@ const char *msd_error_string(int code);
  */
 int msd_init(void *stream);
 
-/* Frees every scratch buffer created so far on all devices. */
+/* Frees every scratch buffer created so far on all devices.  Call it only when no
+ * msd_groupnorm* launch is still in flight (synchronise the streams first); the next
+ * GroupNorm creates its scratch again. */
 int msd_shutdown(void);
 
 /*
@@ -60,7 +62,8 @@ int msd_status(void *stream);
 
 /*
  * Tuning / test knobs (process-wide; value 0 restores the automatic choice).  They change
- * how a launch is cut into workgroups, never its result.  No reference counterpart.
+ * how a launch is cut into workgroups, never its result.  Plain globals: set them while no
+ * other thread is launching.  No reference counterpart.
  */
 #define MSD_TUNE_GN_SPLIT 0      /* workgroups per (sample, group): power of two <= 64 */
 #define MSD_TUNE_GN_THREADS 1    /* GroupNorm workgroup size: multiple of 64, <= 1024 */
