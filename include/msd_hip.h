@@ -238,6 +238,7 @@ int msd_softmax(const void *x, void *y, size_t rows, size_t cols, int stable, in
  *                       + sqrt(1 - a_prev) * e_t, the three loops of p_sample_ddim (:107-118,
  *                       eta 0) in one pass, every operation rounded separately in that order
  *                       (bit-identical to the host loops for float32).  x_prev may alias x.
+ *                       a_t must be > 0 and a_prev in [0, 1] (else invalid value).
  */
 int msd_alphas_cumprod(float *out_1000);
 int msd_ddim_schedule(int ddim_num_steps, int *timesteps, float *alphas, float *alphas_prev,

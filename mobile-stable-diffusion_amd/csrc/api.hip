@@ -362,6 +362,7 @@ int msd_ddim_update(const void *x, const void *e_t, void *x_prev, size_t n, floa
                     float a_prev, float sqrt_one_minus_at, int dtype, void *stream) {
     if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
     if (n != 0 && (!x || !e_t || !x_prev)) return MSD_ERR_INVALID_VALUE;
+    if (!(a_t > 0.0f) || !(a_prev >= 0.0f) || !(a_prev <= 1.0f)) return MSD_ERR_INVALID_VALUE;  // sqrt / division
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == MSD_DTYPE_F32)
         return ddim_update_dispatch<float>(x, e_t, x_prev, n, a_t, a_prev, sqrt_one_minus_at, s);

@@ -72,8 +72,22 @@ def test_argument_validation_needs_no_gpu(msd):
     assert lib.msd_set_tuning(0, 3) == 1      # split must be a power of two
     assert lib.msd_set_tuning(1, 100) == 1    # threads must be a multiple of 64
     assert lib.msd_set_tuning(2, 12) == 1 and lib.msd_set_tuning(4, 3) == 1 and lib.msd_set_tuning(99, 1) == 1
-    for knob in range(6):
+    assert lib.msd_set_tuning(6, 48) == 1     # softmax rows per workgroup: 16, 32 or 64
+    for knob in range(7):
         assert lib.msd_set_tuning(knob, 0) == 0
+    # the neighbours of the path
+    assert lib.msd_linear_rows(None, None, None, None, 9, 4, 8, 0, 0, 0, None) == 1   # more than 8 rows
+    assert lib.msd_linear_rows(None, None, None, None, 2, 4, 8, 0, 0, 0, None) == 1   # null pointers
+    assert lib.msd_linear_rows(None, None, None, None, 2, 4, 8, 3, 0, 0, None) == 1   # unknown activation
+    assert lib.msd_softmax(None, None, 4, 77, 0, 0, None) == 1
+    assert lib.msd_softmax(None, None, 0, 77, 0, 0, None) == 0                        # empty: nothing to do
+    assert lib.msd_ddim_update(None, None, None, 16, 0.5, 0.5, 0.7, 0, None) == 1
+    one = ctypes.c_void_p(16)  # never dereferenced: the coefficients are rejected first
+    assert lib.msd_ddim_update(one, one, one, 16, 0.0, 0.5, 0.7, 0, None) == 1        # a_t must be > 0
+    assert lib.msd_ddim_update(one, one, one, 16, 0.5, 1.5, 0.7, 0, None) == 1        # a_prev in [0, 1]
+    assert lib.msd_alphas_cumprod(None) == 1
+    assert lib.msd_ddim_schedule(50, None, None, None, None, 0) == 50
+    assert lib.msd_ddim_schedule(501, None, None, None, None, 0) == -2
 
 
 def test_missing_library_fails_loudly(msd):
