@@ -8,7 +8,7 @@ each layer on its own HBM-resident buffers, launched back to back on one stream.
 `value` = algorithmic bytes of one step / time per step.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode graph|eager]
-                    [--no-cpu] [--no-shapes] [--tables shapes,fusions,neighbours,large_batch]
+                    [--no-cpu] [--no-shapes] [--tables shapes,fusions,neighbours,large_batch,gn_split]
 
 Prints ONE JSON line (see the keys below).  The CPU oracle is used only for the
 `cpu_baseline` leg.
@@ -25,9 +25,18 @@ if REPO not in sys.path:
     sys.path.insert(0, REPO)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
-# measured HBM bytes per geglu_kernel<__half> launch, averaged over the 16 launches of a step
-# (rocprofv3 counters; algorithmic figure is 34652160)
-GEGLU_TRAFFIC_BYTES_PER_LAUNCH = 34683383
+# HBM bytes per launch of each kernel family as the rocprofv3 FETCH_SIZE / WRITE_SIZE counters
+# measured them (written next to the counter summary it was computed from)
+TRAFFIC_JSON = os.path.join(REPO, "profiles", "traffic.json")
+
+
+def measured_traffic():
+    """{family: HBM bytes per launch} from profiles/traffic.json; {} when the file is absent."""
+    try:
+        with open(TRAFFIC_JSON) as f:
+            return {k: v.get("traffic_bytes_per_launch") for k, v in json.load(f)["families"].items()}
+    except (OSError, ValueError, KeyError):
+        return {}
 
 
 # ----------------------------------------------------------------------------
@@ -233,78 +242,141 @@ def capture(torch, msd, stream, body):
     return graph.replay
 
 
-def shape_table(torch, msd, dev, stream):
-    """Per-kernel µs / GB/s / % of HBM peak at the UNet shapes, fp16 and fp32, each launch on
-    its own buffers (rotating over > 600 MB so nothing is cache-resident), graph-replayed."""
+def _rotating_launch_us(torch, msd, stream, launch, xs, ys, warm=20, budget=2000):
+    """µs per launch of `launch(x, y, stream_ptr)` over rotating buffer pairs, graph-replayed."""
+    import ctypes
+    copies = len(xs)
+
+    def body():
+        sp = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        for x, y in zip(xs, ys):
+            assert launch(x, y, sp) == 0
+    replay = capture(torch, msd, stream, body)
+    reps = max(2, int(budget // copies))
+    with torch.cuda.stream(stream):
+        for _ in range(warm // copies + 1):  # at least `warm` warm-up launches
+            replay()
+        return event_time_ms(torch, replay, reps) * 1e3 / (reps * copies)
+
+
+def _kernel_case(torch, msd, dev, kind, p, dt, batch):
+    """Buffers, launch closure and byte counts for one row of the per-kernel tables."""
     import ctypes
     vp = ctypes.c_void_p
     lib = msd.load_library()
-    rows = []
-    cases = []
+    code, elt = (msd.DTYPE_F16, 2) if dt == torch.float16 else (msd.DTYPE_F32, 4)
+    if kind == "groupnorm_silu":
+        n_in = n_out = batch * p["c"] * p["hw"]
+        nbytes = 2 * n_in * elt
+    elif kind == "layernorm":
+        n_in = n_out = p["rows"] * p["dim"]
+        nbytes = 2 * n_in * elt
+    elif kind == "geglu":
+        n_in, n_out = 2 * p["rows"] * p["inner"], p["rows"] * p["inner"]
+        nbytes = 3 * n_out * elt
+    else:  # elementwise activation
+        n_in = n_out = p["n"]
+        nbytes = 2 * n_in * elt
+    copies = max(4, min(256, int(640e6 // max(nbytes, 1)) + 1))
+    xs = [torch.randn(n_in, device=dev, dtype=torch.float32).to(dt) for _ in range(copies)]
+    ys = [torch.empty(n_out, device=dev, dtype=dt) for _ in range(copies)]
+    cdim = p.get("c", p.get("dim", 1))
+    ga = torch.ones(cdim, device=dev)
+    be = torch.zeros(cdim, device=dev)
+
+    def launch(x, y, sp):
+        if kind == "groupnorm_silu":
+            return lib.msd_groupnorm(vp(x.data_ptr()), vp(y.data_ptr()), vp(ga.data_ptr()), vp(be.data_ptr()),
+                                     batch, p["c"], p["hw"], 32, 1e-5, 1, code, sp)
+        if kind == "layernorm":
+            return lib.msd_layernorm(vp(x.data_ptr()), vp(y.data_ptr()), vp(ga.data_ptr()), vp(be.data_ptr()),
+                                     p["rows"], p["dim"], 1e-5, code, sp)
+        if kind == "geglu":
+            return lib.msd_geglu(vp(x.data_ptr()), vp(y.data_ptr()), p["rows"], p["inner"], code, sp)
+        return getattr(lib, "msd_" + kind)(vp(x.data_ptr()), vp(y.data_ptr()), p["n"], code, sp)
+
+    def copy_launch(x, y, sp):  # the same bytes through the plain copy kernel
+        return lib.msd_copy(vp(x.data_ptr()), vp(y.data_ptr()), n_out * elt, sp)
+    return {"xs": xs, "ys": ys, "keep": (ga, be), "launch": launch, "copy_launch": copy_launch,
+            "bytes": nbytes, "copy_same_bytes": n_in == n_out, "elt": elt}
+
+
+def shape_table(torch, msd, dev, stream):
+    """Per-kernel µs / GB/s / % of HBM peak at the shapes of BASELINE configs 1 - 4, each launch
+    on its own buffers (rotating over > 600 MB so nothing is cache-resident), graph-replayed,
+    next to a plain copy of the same bytes.  Config 2 / 3 at batch 2 in fp16 (GroupNorm also
+    fp32); config 1 (one fp32 tensor) and config 4 (text-encoder shapes, fp32) are a few hundred
+    KB to 10 MB per launch and are bound by the launch floor, not by bandwidth."""
+    f16, f32 = torch.float16, torch.float32
+    cases = [("cfg1", "groupnorm_silu", {"c": 320, "hw": 4096}, f32, 1)]
     for c, side in [(320, 64), (640, 32), (1280, 16), (1280, 8), (960, 32), (1920, 16)]:
-        cases.append(("groupnorm_silu", {"c": c, "hw": side * side}))
+        cases.append(("cfg2", "groupnorm_silu", {"c": c, "hw": side * side}, f16, BATCH))
+        cases.append(("cfg2", "groupnorm_silu", {"c": c, "hw": side * side}, f32, BATCH))
     for r, d in [(8192, 320), (2048, 640), (512, 1280)]:
-        cases.append(("layernorm", {"rows": r, "dim": d}))
+        cases.append(("cfg3", "layernorm", {"rows": r, "dim": d}, f16, BATCH))
     for r, i in [(8192, 1280), (2048, 2560), (512, 5120)]:
-        cases.append(("geglu", {"rows": r, "inner": i}))
-    for kind, p in cases:
-        for dt, code, elt in ((torch.float16, msd.DTYPE_F16, 2), (torch.float32, msd.DTYPE_F32, 4)):
-            if kind != "groupnorm_silu" and dt == torch.float32:
-                continue
-            if kind == "groupnorm_silu":
-                n_in = n_out = BATCH * p["c"] * p["hw"]
-                nbytes = 2 * n_in * elt
-            elif kind == "layernorm":
-                n_in = n_out = p["rows"] * p["dim"]
-                nbytes = 2 * n_in * elt
-            else:
-                n_in, n_out = 2 * p["rows"] * p["inner"], p["rows"] * p["inner"]
-                nbytes = 3 * n_out * elt
-            copies = max(4, min(256, int(640e6 // nbytes) + 1))
-            xs = [torch.randn(n_in, device=dev, dtype=torch.float32).to(dt) for _ in range(copies)]
-            ys = [torch.empty(n_out, device=dev, dtype=dt) for _ in range(copies)]
-            cdim = p.get("c", p.get("dim", 1))
-            ga = torch.ones(cdim, device=dev)
-            be = torch.zeros(cdim, device=dev)
+        cases.append(("cfg3", "geglu", {"rows": r, "inner": i}, f16, BATCH))
+    cases.append(("cfg4", "layernorm", {"rows": 77, "dim": 768}, f32, 1))
+    cases.append(("cfg4", "layernorm", {"rows": 154, "dim": 768}, f32, 2))
+    cases.append(("cfg4", "quick_gelu", {"n": 2 * 77 * 3072}, f32, 2))
+    rows = []
+    for cfg, kind, p, dt, batch in cases:
+        case = _kernel_case(torch, msd, dev, kind, p, dt, batch)
+        us = _rotating_launch_us(torch, msd, stream, case["launch"], case["xs"], case["ys"])
+        gbs = case["bytes"] / us / 1e3
+        row = {"config": cfg, "kernel": kind, "shape": dict(p, batch=batch), "dtype": "f16" if case["elt"] == 2 else "f32",
+               "bytes": case["bytes"], "us": round(us, 3), "GBps": round(gbs, 1),
+               "pct_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 1)}
+        if case["copy_same_bytes"]:  # one copy launch moves exactly the kernel's bytes
+            cus = _rotating_launch_us(torch, msd, stream, case["copy_launch"], case["xs"], case["ys"])
+            row["copy_us"] = round(cus, 3)
+            row["pct_of_copy_rate"] = round(100.0 * cus / us, 1)
+        if cfg in ("cfg1", "cfg4"):
+            row["note"] = "launch-bound: %.2f us at 8 TB/s" % (case["bytes"] / HBM_PEAK_GBS / 1e3)
+        rows.append(row)
+        del case
+        torch.cuda.empty_cache()
+    return rows
 
-            def body():
-                sp = vp(torch.cuda.current_stream().cuda_stream)
-                for x, y in zip(xs, ys):
-                    if kind == "groupnorm_silu":
-                        rc = lib.msd_groupnorm(vp(x.data_ptr()), vp(y.data_ptr()), vp(ga.data_ptr()),
-                                               vp(be.data_ptr()), BATCH, p["c"], p["hw"], 32, 1e-5, 1, code, sp)
-                    elif kind == "layernorm":
-                        rc = lib.msd_layernorm(vp(x.data_ptr()), vp(y.data_ptr()), vp(ga.data_ptr()),
-                                               vp(be.data_ptr()), p["rows"], p["dim"], 1e-5, code, sp)
-                    else:
-                        rc = lib.msd_geglu(vp(x.data_ptr()), vp(y.data_ptr()), p["rows"], p["inner"], code, sp)
-                    assert rc == 0
-            # the same bytes through a plain copy kernel: what a launch of this size can reach
-            in_bytes, out_bytes = n_in * elt, n_out * elt
 
-            def copy_body():
-                sp = vp(torch.cuda.current_stream().cuda_stream)
-                for x, y in zip(xs, ys):
-                    assert lib.msd_copy(vp(x.data_ptr()), vp(y.data_ptr()), out_bytes, sp) == 0
-            reps = max(2, int(2000 // copies))
-            us = {}
-            for name, fn in (("kernel", body), ("copy", copy_body)):
-                if name == "copy" and in_bytes != out_bytes:
-                    continue
-                replay = capture(torch, msd, stream, fn)
-                with torch.cuda.stream(stream):
-                    for _ in range(20 // copies + 1):  # at least 20 warm-up launches
-                        replay()
-                    us[name] = event_time_ms(torch, replay, reps) * 1e3 / (reps * copies)
-            gbs = nbytes / us["kernel"] / 1e3
-            row = {"kernel": kind, "shape": p, "dtype": "f16" if elt == 2 else "f32",
-                   "bytes": nbytes, "us": round(us["kernel"], 3), "GBps": round(gbs, 1),
-                   "pct_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 1)}
-            if in_bytes == out_bytes:  # one copy launch moves exactly the kernel's bytes
-                row["copy_us"] = round(us["copy"], 3)
-                row["pct_of_copy_rate"] = round(100.0 * us["copy"] / us["kernel"], 1)
-            rows.append(row)
-            del xs, ys
+def launch_floor_us(torch, msd, dev, stream):
+    """µs per launch of a chain of 16-byte copies replayed as a graph: what one more kernel in
+    a captured step costs when it moves nothing."""
+    import ctypes
+    vp = ctypes.c_void_p
+    lib = msd.load_library()
+    xs = [torch.zeros(4, device=dev) for _ in range(64)]
+    ys = [torch.zeros(4, device=dev) for _ in range(64)]
+    return _rotating_launch_us(torch, msd, stream,
+                               lambda x, y, sp: lib.msd_copy(vp(x.data_ptr()), vp(y.data_ptr()), 16, sp), xs, ys,
+                               budget=20000)
+
+
+def gn_split_table(torch, msd, dev, stream):
+    """GroupNorm+SiLU at the config-2 shapes with the launch plan forced: workgroups per
+    (sample, group) in {1, 2, 4, 8} x workgroup size in {512, 1024}, next to the automatic
+    plan.  `auto_vs_best` > 1.03 would mean the plan in groupnorm.hip picks a slow variant."""
+    lib = msd.load_library()
+    rows = []
+    for c, side in [(320, 64), (640, 32), (1280, 16), (1280, 8), (960, 32), (1920, 16)]:
+        for dt in (torch.float16, torch.float32):
+            case = _kernel_case(torch, msd, dev, "groupnorm_silu", {"c": c, "hw": side * side}, dt, BATCH)
+            times = {}
+            try:
+                for split in (0, 1, 2, 4, 8):
+                    for threads in ((0,) if split == 0 else (512, 1024)):
+                        assert lib.msd_set_tuning(msd.TUNE_GN_SPLIT, split) == 0
+                        assert lib.msd_set_tuning(msd.TUNE_GN_THREADS, threads) == 0
+                        key = "auto" if split == 0 else "s%d_t%d" % (split, threads)
+                        times[key] = round(_rotating_launch_us(torch, msd, stream, case["launch"], case["xs"],
+                                                               case["ys"], budget=1000), 3)
+            finally:
+                lib.msd_set_tuning(msd.TUNE_GN_SPLIT, 0)
+                lib.msd_set_tuning(msd.TUNE_GN_THREADS, 0)
+            best = min(v for k, v in times.items() if k != "auto")
+            rows.append({"shape": {"c": c, "hw": side * side, "batch": BATCH}, "dtype": "f16" if case["elt"] == 2 else "f32",
+                         "us": times, "best_forced_us": best, "auto_vs_best": round(times["auto"] / best, 3)})
+            del case
             torch.cuda.empty_cache()
     return rows
 
@@ -711,7 +783,8 @@ def cpu_baseline(total_bytes, budget_s=24.0):
             "ms_per_step": round(per_step * 1e3, 2), "seconds_timed": round(t_total, 2),
             "sample": "the layers of one full UNet step (45 GN+SiLU, 48 LN, 16 GEGLU, 23 SiLU, 1 embedding), "
                       "%d repetitions each, fp32, unfused passes as the reference enqueues them, OpenMP over "
-                      "groups/rows; GB/s uses the same fp16 algorithmic bytes as the GPU figure" % reps}
+                      "groups/rows; GB/s uses the same fp16 algorithmic bytes as the GPU figure; oracle built "
+                      "with %s" % (reps, orc.build_flags())}
 
 
 def main():
@@ -723,7 +796,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-kernel tables")
     ap.add_argument("--tables", default="shapes,fusions,neighbours,large_batch",
-                    help="comma list of the per-kernel tables to measure")
+                    help="comma list of the per-kernel tables to measure (also: gn_split, the forced "
+                         "launch-plan sweep of GroupNorm)")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="for rocprofv3 --pmc runs: one 64 MiB device copy (known traffic) then three "
                          "eager steps; prints nothing")
@@ -801,16 +875,24 @@ def main():
                               "us_per_launch": round(ms * 1e3 / k["launches"], 3), "GBps": round(gbs, 1),
                               "pct_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 1)}
 
-    # The kernel with the largest total GPU time in the rocprofv3 kernel statistics of this
-    # workload is geglu_kernel<__half> (the GroupNorm time is spread over several template
-    # instances).  Its live figure comes from the HIP-event timing above; its HBM traffic per
-    # launch was measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, calibrated on a plain
-    # 64 MiB copy (FETCH_SIZE x 1.9992, WRITE_SIZE x 1.0000).
-    dk = families["geglu"]
-    roofline = {"bound": "hbm", "kernel": "geglu_kernel<__half, 1>", "achieved": dk["GBps"], "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": round(dk["GBps"] / HBM_PEAK_GBS, 4),
-                "bytes_per_launch": dk["bytes"] // dk["launches"], "us_per_launch": dk["us_per_launch"],
-                "traffic": GEGLU_TRAFFIC_BYTES_PER_LAUNCH}
+    # One block per kernel family: algorithmic bytes per launch / live HIP-event time per launch
+    # against the 8 TB/s peak, with the HBM traffic per launch that rocprofv3 --pmc FETCH_SIZE /
+    # WRITE_SIZE measured (profiles/traffic.json).  `roofline` is the single kernel with the
+    # largest total GPU time in the rocprofv3 kernel statistics of this workload,
+    # geglu_kernel<__half, 1>; the GroupNorm family as a whole takes more of the step and sits
+    # furthest below the roofline, which `roofline_families` shows.
+    traffic = measured_traffic()
+    kernel_names = {"gn_silu": "gn_slice_kernel<__half, K, true>", "ln": "ln_team_kernel<__half, NW, VPL, TL>",
+                    "geglu": "geglu_kernel<__half, 1>"}
+    roofline_families = {}
+    for kind, fam in families.items():
+        roofline_families[kind] = {
+            "bound": "hbm", "kernel": kernel_names[kind], "achieved": fam["GBps"], "peak": HBM_PEAK_GBS,
+            "unit": "GB/s", "frac": round(fam["GBps"] / HBM_PEAK_GBS, 4), "launches_per_step": fam["launches"],
+            "bytes_per_launch": fam["bytes"] // fam["launches"], "us_per_launch": fam["us_per_launch"],
+            "pct_of_step_time": round(100 * fam["us_total"] / (ms_per_step * 1e3), 1),
+            "traffic": traffic.get(kind)}
+    roofline = dict(roofline_families["geglu"])
 
     out = {
         "metric": "fused GroupNorm+SiLU/LayerNorm/GEGLU HBM GB/s over one SD UNet step (batch 2, fp16 storage)",
@@ -823,8 +905,10 @@ def main():
                    "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 1),
                    "copy_step_ms": round(copy_ms, 4), "pct_of_copy_step_rate": round(100 * copy_ms / ms_per_step, 1)},
         "roofline": roofline,
+        "roofline_families": roofline_families,
         "kernel_families": families,
     }
+    out["config"]["launch_floor_us"] = round(launch_floor_us(torch, msd, dev, stream), 3)
     tables = set() if args.no_shapes else set(t for t in args.tables.split(",") if t)
     if "shapes" in tables:
         out["shapes"] = shape_table(torch, msd, dev, stream)
@@ -834,6 +918,8 @@ def main():
         out["step_with_adds"] = step_with_adds(torch, msd, dev, stream)
     if "large_batch" in tables:
         out["large_batch"] = large_batch_table(torch, msd, dev, stream)
+    if "gn_split" in tables:
+        out["gn_split"] = gn_split_table(torch, msd, dev, stream)
     if "neighbours" in tables:
         out["neighbours"] = neighbour_table(torch, msd, dev, stream)
     if not args.no_cpu:

@@ -43,10 +43,15 @@ const char *msd_error_string(int code);
  * stream capture.  A graph captured on a stream keeps using that stream's
  * scratch: GroupNorm launches that share scratch must not run concurrently
  * (do not replay such a graph on a second stream while the first is busy with
- * GroupNorms).  No reference counterpart (the reference allocates two
- * temporaries per forward, M/nn/GroupNorm.cpp:95-103).
+ * GroupNorms).  hipStreamPerThread is refused (one handle, a
+ * different stream in every thread).  No reference counterpart (the reference
+ * allocates two temporaries per forward, M/nn/GroupNorm.cpp:95-103).
  */
 int msd_init(void *stream);
+
+/* Frees the scratch of `stream` on the current device (for applications that create and
+ * destroy streams; the stream must be idle).  The next GroupNorm on it creates it again. */
+int msd_release(void *stream);
 
 /* Frees every scratch buffer created so far on all devices.  Call it only when no
  * msd_groupnorm* launch is still in flight (synchronise the streams first); the next
@@ -54,16 +59,25 @@ int msd_init(void *stream);
 int msd_shutdown(void);
 
 /*
- * Synchronises `stream` and reports whether any msd_groupnorm launched on it
- * so far gave up waiting for a sibling workgroup (its output is then invalid):
- * 0, or hipErrorLaunchFailure.  The flag is sticky.  No reference counterpart.
+ * Synchronises `stream`; returns 0 or the HIP error the stream reports.  No reference
+ * counterpart (the reference blocks in clFinish, M/UNetModel.cpp:1830).
  */
 int msd_status(void *stream);
 
 /*
+ * Diagnostic.  Workgroups that share one (sample, group) exchange partial statistics; one
+ * that does not receive a sibling's within its poll limit computes them itself from the
+ * input, so the output is right either way.  This synchronises `stream` and returns in
+ * *count how often that happened so far on the stream's scratch (0 on an idle GPU);
+ * reset != 0 clears the counter.
+ */
+int msd_gn_fallbacks(void *stream, unsigned int *count, int reset);
+
+/*
  * Tuning / test knobs (process-wide; value 0 restores the automatic choice).  They change
- * how a launch is cut into workgroups, never its result.  Plain globals: set them while no
- * other thread is launching.  No reference counterpart.
+ * how a launch is cut into workgroups, never its result.  Each launch reads a knob once
+ * (atomically), so setting one while another thread launches is safe but affects that
+ * thread's later launches.  No reference counterpart.
  */
 #define MSD_TUNE_GN_SPLIT 0      /* workgroups per (sample, group): power of two <= 64 */
 #define MSD_TUNE_GN_THREADS 1    /* GroupNorm workgroup size: multiple of 64, <= 1024 */
@@ -72,6 +86,8 @@ int msd_status(void *stream);
 #define MSD_TUNE_GEGLU_VECTORS 4 /* 16-byte vectors per GEGLU lane: 1, 2 or 4 */
 #define MSD_TUNE_ACT_VECTORS 5   /* 16-byte vectors per lane of SiLU / GELU / quick_GELU: 1, 2 or 4 */
 #define MSD_TUNE_SOFTMAX_ROWS 6   /* rows per workgroup of the short-row softmax: 16, 32 or 64 */
+#define MSD_TUNE_GN_SPIN_LIMIT 7  /* polls a GroupNorm workgroup waits for a sibling before it computes
+                                     that sibling's statistics itself (tests set 1 to exercise that path) */
 int msd_set_tuning(int knob, int value);
 
 /*

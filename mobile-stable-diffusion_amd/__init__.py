@@ -18,12 +18,12 @@ LIB_NN_PATH = os.path.join(CSRC_DIR, "libmsd_nn.so")
 DTYPE_F32 = 0
 DTYPE_F16 = 1
 TUNE_GN_SPLIT, TUNE_GN_THREADS, TUNE_LN_CHUNK, TUNE_LN_THREADS, TUNE_GEGLU_VECTORS, TUNE_ACT_VECTORS, \
-    TUNE_SOFTMAX_ROWS = range(7)
+    TUNE_SOFTMAX_ROWS, TUNE_GN_SPIN_LIMIT = range(8)
 
 # every symbol include/msd_hip.h declares
 C_ABI_SYMBOLS = (
-    "msd_version", "msd_error_string", "msd_init", "msd_shutdown", "msd_status",
-    "msd_set_tuning", "msd_groupnorm", "msd_layernorm", "msd_geglu",
+    "msd_version", "msd_error_string", "msd_init", "msd_release", "msd_shutdown", "msd_status",
+    "msd_gn_fallbacks", "msd_set_tuning", "msd_groupnorm", "msd_layernorm", "msd_geglu",
     "msd_silu", "msd_gelu", "msd_quick_gelu", "msd_timestep_embedding", "msd_ddim_timesteps",
     "msd_elemwise_add", "msd_chunkwise_add", "msd_chunk_add_groupnorm", "msd_add_layernorm", "msd_copy",
     "msd_groupnorm_tokens", "msd_permute_0_2_1",
@@ -56,6 +56,8 @@ def load_library(path=None):
     lib.msd_init.argtypes = [vp]
     lib.msd_shutdown.argtypes = []
     lib.msd_status.argtypes = [vp]
+    lib.msd_release.argtypes = [vp]
+    lib.msd_gn_fallbacks.argtypes = [vp, ctypes.POINTER(ctypes.c_uint), it]
     lib.msd_set_tuning.argtypes = [it, it]
     lib.msd_groupnorm.argtypes = [vp, vp, vp, vp, sz, sz, sz, sz, fl, it, it, vp]
     lib.msd_layernorm.argtypes = [vp, vp, vp, vp, sz, sz, fl, it, vp]
@@ -110,6 +112,23 @@ def _dev(t):
     return ctypes.c_void_p(t.data_ptr())
 
 
+def _affine(t, n, like, what):
+    """gamma / beta / bias: float32, n values, on the device of `like`."""
+    import torch
+    if t.dtype != torch.float32 or t.numel() != n or t.device != like.device:
+        raise MsdError("%s must be float32 with %d values on %s (got %s, %d, %s)"
+                       % (what, n, like.device, t.dtype, t.numel(), t.device))
+    return _dev(t)
+
+
+def _same(t, like, numel, what):
+    """An output / second operand: dtype and device of `like`, `numel` elements."""
+    if t.dtype != like.dtype or t.device != like.device or t.numel() != numel:
+        raise MsdError("%s must be %s with %d elements on %s (got %s, %d, %s)"
+                       % (what, like.dtype, numel, like.device, t.dtype, t.numel(), t.device))
+    return _dev(t)
+
+
 def init():
     check(load_library().msd_init(_stream()))
 
@@ -118,14 +137,23 @@ def status():
     return load_library().msd_status(_stream())
 
 
+def gn_fallbacks(reset=False):
+    """How often a GroupNorm workgroup computed a sibling's statistics itself (diagnostic)."""
+    n = ctypes.c_uint(0)
+    check(load_library().msd_gn_fallbacks(_stream(), ctypes.byref(n), int(reset)))
+    return n.value
+
+
 def groupnorm(x, gamma, beta, groups, eps=1e-5, fuse_silu=False, out=None):
     """x: [batch, C, ...] device tensor; gamma/beta float32 [C]; out may be x (in place)."""
     import torch
     out = torch.empty_like(x) if out is None else out
     batch, channels = x.shape[0], x.shape[1]
     hw = x.numel() // (batch * channels) if batch * channels else 0
-    check(load_library().msd_groupnorm(_dev(x), _dev(out), _dev(gamma), _dev(beta), batch, channels,
-                                       hw, groups, eps, int(fuse_silu), _dtype_code(x), _stream()))
+    fn = load_library().msd_groupnorm
+    check(fn(_dev(x), _same(out, x, x.numel(), "out"), _affine(gamma, channels, x, "gamma"),
+             _affine(beta, channels, x, "beta"), batch, channels, hw, groups, eps, int(fuse_silu),
+             _dtype_code(x), _stream()))
     return out
 
 
@@ -135,7 +163,8 @@ def groupnorm_tokens(x, gamma, beta, groups, eps=1e-6):
     batch, channels = x.shape[0], x.shape[1]
     hw = x.numel() // (batch * channels) if batch * channels else 0
     out = torch.empty((batch, hw, channels), dtype=x.dtype, device=x.device)
-    check(load_library().msd_groupnorm_tokens(_dev(x), _dev(out), _dev(gamma), _dev(beta), batch, channels,
+    check(load_library().msd_groupnorm_tokens(_dev(x), _dev(out), _affine(gamma, channels, x, "gamma"),
+                                              _affine(beta, channels, x, "beta"), batch, channels,
                                               hw, groups, eps, _dtype_code(x), _stream()))
     return out
 
@@ -155,7 +184,9 @@ def chunk_add_groupnorm(x, chunk, gamma, beta, groups, eps=1e-5, fuse_silu=False
     out = torch.empty_like(x) if out is None else out
     batch, channels = x.shape[0], x.shape[1]
     hw = x.numel() // (batch * channels) if batch * channels else 0
-    check(load_library().msd_chunk_add_groupnorm(_dev(x), _dev(chunk), _dev(out), _dev(gamma), _dev(beta),
+    check(load_library().msd_chunk_add_groupnorm(_dev(x), _same(chunk, x, batch * channels, "chunk"),
+                                                 _same(out, x, x.numel(), "out"),
+                                                 _affine(gamma, channels, x, "gamma"), _affine(beta, channels, x, "beta"),
                                                  batch, channels, hw, groups, eps, int(fuse_silu),
                                                  _dtype_code(x), _stream()))
     return out
@@ -168,22 +199,27 @@ def add_layernorm(a, b, gamma, beta, eps=1e-5, sum_out=None, out=None):
     out = torch.empty_like(a) if out is None else out
     dim = a.shape[-1]
     rows = a.numel() // dim if dim else 0
-    check(load_library().msd_add_layernorm(_dev(a), _dev(b), _dev(sum_out), _dev(out), _dev(gamma),
-                                           _dev(beta), rows, dim, eps, _dtype_code(a), _stream()))
+    check(load_library().msd_add_layernorm(_dev(a), _same(b, a, a.numel(), "b"), _same(sum_out, a, a.numel(), "sum_out"),
+                                           _same(out, a, a.numel(), "out"), _affine(gamma, dim, a, "gamma"),
+                                           _affine(beta, dim, a, "beta"), rows, dim, eps, _dtype_code(a), _stream()))
     return sum_out, out
 
 
 def elemwise_add(a, b, out=None):
     import torch
     out = torch.empty_like(a) if out is None else out
-    check(load_library().msd_elemwise_add(_dev(a), _dev(b), _dev(out), a.numel(), _dtype_code(a), _stream()))
+    check(load_library().msd_elemwise_add(_dev(a), _same(b, a, a.numel(), "b"), _same(out, a, a.numel(), "out"),
+                                          a.numel(), _dtype_code(a), _stream()))
     return out
 
 
 def chunkwise_add(a, chunk, chunk_size, out=None):
     import torch
     out = torch.empty_like(a) if out is None else out
-    check(load_library().msd_chunkwise_add(_dev(a), _dev(chunk), _dev(out), a.numel(), chunk_size,
+    if chunk_size <= 0 or a.numel() % chunk_size:
+        raise MsdError("chunk_size must divide the element count")
+    check(load_library().msd_chunkwise_add(_dev(a), _same(chunk, a, a.numel() // chunk_size, "chunk"),
+                                           _same(out, a, a.numel(), "out"), a.numel(), chunk_size,
                                            _dtype_code(a), _stream()))
     return out
 
@@ -193,7 +229,8 @@ def layernorm(x, gamma, beta, eps=1e-5, out=None):
     out = torch.empty_like(x) if out is None else out
     dim = x.shape[-1]
     rows = x.numel() // dim if dim else 0
-    check(load_library().msd_layernorm(_dev(x), _dev(out), _dev(gamma), _dev(beta), rows, dim, eps,
+    check(load_library().msd_layernorm(_dev(x), _same(out, x, x.numel(), "out"), _affine(gamma, dim, x, "gamma"),
+                                       _affine(beta, dim, x, "beta"), rows, dim, eps,
                                        _dtype_code(x), _stream()))
     return out
 
@@ -205,14 +242,16 @@ def geglu(proj, out=None):
     rows = proj.numel() // (2 * inner) if inner else 0
     if out is None:
         out = torch.empty(proj.shape[:-1] + (inner,), dtype=proj.dtype, device=proj.device)
-    check(load_library().msd_geglu(_dev(proj), _dev(out), rows, inner, _dtype_code(proj), _stream()))
+    check(load_library().msd_geglu(_dev(proj), _same(out, proj, rows * inner, "out"), rows, inner,
+                                   _dtype_code(proj), _stream()))
     return out
 
 
 def _act(name, x, out):
     import torch
     out = torch.empty_like(x) if out is None else out
-    check(getattr(load_library(), name)(_dev(x), _dev(out), x.numel(), _dtype_code(x), _stream()))
+    check(getattr(load_library(), name)(_dev(x), _same(out, x, x.numel(), "out"), x.numel(), _dtype_code(x),
+                                        _stream()))
     return out
 
 
@@ -257,8 +296,10 @@ def linear_rows(x, weight, bias=None, act_in=ACT_NONE, act_out=ACT_NONE, out=Non
     if weight.shape[1] != k or weight.dtype != x.dtype:
         raise MsdError("weight must be [n, k] in the dtype of x")
     out = torch.empty((m, n), dtype=x.dtype, device=x.device) if out is None else out
-    bp = _dev(bias) if bias is not None else None
-    check(load_library().msd_linear_rows(_dev(x), _dev(weight), bp, _dev(out), m, n, k, act_in, act_out,
+    if weight.device != x.device:
+        raise MsdError("weight and x must share a device")
+    bp = _affine(bias, n, x, "bias") if bias is not None else None
+    check(load_library().msd_linear_rows(_dev(x), _dev(weight), bp, _same(out, x, m * n, "out"), m, n, k, act_in, act_out,
                                          _dtype_code(x), _stream()))
     return out
 
@@ -269,7 +310,8 @@ def softmax(x, stable=False, out=None):
     out = torch.empty_like(x) if out is None else out
     cols = x.shape[-1]
     rows = x.numel() // cols if cols else 0
-    check(load_library().msd_softmax(_dev(x), _dev(out), rows, cols, int(stable), _dtype_code(x), _stream()))
+    check(load_library().msd_softmax(_dev(x), _same(out, x, x.numel(), "out"), rows, cols, int(stable),
+                                     _dtype_code(x), _stream()))
     return out
 
 
@@ -296,7 +338,8 @@ def ddim_update(x, e_t, a_t, a_prev, sqrt_one_minus_at, out=None):
     """One DDIM step (eta 0) on device tensors; out may be x."""
     import torch
     out = torch.empty_like(x) if out is None else out
-    check(load_library().msd_ddim_update(_dev(x), _dev(e_t), _dev(out), x.numel(), a_t, a_prev,
+    check(load_library().msd_ddim_update(_dev(x), _same(e_t, x, x.numel(), "e_t"), _same(out, x, x.numel(), "out"),
+                                         x.numel(), a_t, a_prev,
                                          sqrt_one_minus_at, _dtype_code(x), _stream()))
     return out
 
@@ -360,7 +403,12 @@ def load_nn_library(path=None):
         "msdnn_ddim_sample": (it, [vp, vp, sz, it, it, MODEL_FN, vp, vp]),
         "msdnn_ddim_make_schedule": (it, [ctypes.POINTER(ctypes.c_int), it, flp, flp]),
         "msdnn_test_buffer": (it, [vp, vp, sz, it, cp, flp, szp]),
-        "msdnn_step_create": (vp, [vp, sz, it]),
+        "msdnn_step_create": (vp, [vp, sz, it, it]),
+        "msdnn_step_num_ops": (sz, [vp]),
+        "msdnn_step_op_info": (it, [vp, sz, ctypes.POINTER(ctypes.c_int), szp, ctypes.POINTER(ctypes.c_int)]),
+        "msdnn_step_download": (it, [vp, sz, it, flp, sz, szp]),
+        "msdnn_step_affine": (it, [vp, sz, flp, flp, sz]),
+        "msdnn_step_restore": (it, [vp]),
         "msdnn_step_bytes": (sz, [vp]),
         "msdnn_step_launches": (sz, [vp]),
         "msdnn_step_run": (it, [vp, it, it, lgp, sz]),

@@ -25,15 +25,30 @@ struct ScratchKeyHash {
 std::mutex g_scratch_mutex;
 std::unordered_map<ScratchKey, GnScratch, ScratchKeyHash> g_scratch;
 
-constexpr size_t kSlotBytes = sizeof(unsigned long long) * kGnMaxUnits * kGnMaxSplit;
-constexpr size_t kWordBytes = sizeof(uint32_t) * kGnMaxUnits;
-constexpr size_t kScratchBytes = 2 * kSlotBytes + 2 * kWordBytes + 256;
+// Scratch for `units` (sample, group) pairs, carved out of one block:
+// [slot_mean | slot_m2 | epoch | done | fallbacks], every part 256-byte aligned.
+constexpr size_t slot_bytes(size_t units) { return sizeof(unsigned long long) * units * kGnMaxSplit; }
+constexpr size_t word_bytes(size_t units) { return sizeof(uint32_t) * units; }
+constexpr size_t scratch_bytes(size_t units) { return 2 * slot_bytes(units) + 2 * word_bytes(units) + 256; }
+
+GnScratch carve(char *base, size_t units) {
+    GnScratch s;
+    s.slot_mean = reinterpret_cast<unsigned long long *>(base);
+    s.slot_m2 = reinterpret_cast<unsigned long long *>(base + slot_bytes(units));
+    s.epoch = reinterpret_cast<uint32_t *>(base + 2 * slot_bytes(units));
+    s.done = reinterpret_cast<uint32_t *>(base + 2 * slot_bytes(units) + word_bytes(units));
+    s.fallbacks = reinterpret_cast<uint32_t *>(base + 2 * slot_bytes(units) + 2 * word_bytes(units));
+    s.units = (uint32_t)units;
+    return s;
+}
 
 }  // namespace
 
 // Scratch is private to a (device, stream) pair: launches on one stream are ordered, so a
 // unit's slots are never shared by two launches in flight.
 hipError_t get_scratch(hipStream_t stream, GnScratch *out) {
+    // one handle that names a different stream in every thread cannot key a per-stream scratch
+    if (stream == hipStreamPerThread) return hipErrorInvalidValue;
     int device = 0;
     hipError_t err = hipGetDevice(&device);
     if (err != hipSuccess) return err;
@@ -45,25 +60,23 @@ hipError_t get_scratch(hipStream_t stream, GnScratch *out) {
         return hipSuccess;
     }
     char *base = nullptr;
-    err = hipMalloc(reinterpret_cast<void **>(&base), kScratchBytes);
+    err = hipMalloc(reinterpret_cast<void **>(&base), scratch_bytes(kGnMaxUnits));
     if (err != hipSuccess) return err;
-    err = hipMemset(base, 0, kScratchBytes);  // tags, epochs and counters start at zero
+    err = hipMemset(base, 0, scratch_bytes(kGnMaxUnits));  // tags, epochs and counters start at zero
+    // the fill runs on the null stream: it must have finished before a launch on `stream`
+    // (which may not synchronise with the null stream) reads the scratch
+    if (err == hipSuccess) err = hipStreamSynchronize(nullptr);
     if (err != hipSuccess) {
         (void)hipFree(base);
         return err;
     }
-    GnScratch s;
-    s.slot_mean = reinterpret_cast<unsigned long long *>(base);
-    s.slot_m2 = reinterpret_cast<unsigned long long *>(base + kSlotBytes);
-    s.epoch = reinterpret_cast<uint32_t *>(base + 2 * kSlotBytes);
-    s.done = reinterpret_cast<uint32_t *>(base + 2 * kSlotBytes + kWordBytes);
-    s.status = reinterpret_cast<uint32_t *>(base + 2 * kSlotBytes + 2 * kWordBytes);
+    const GnScratch s = carve(base, kGnMaxUnits);
     g_scratch.emplace(key, s);
     *out = s;
     return hipSuccess;
 }
 
-Tuning g_tuning = {0, 0, 0, 0, 0, 0, 0};
+Tuning g_tuning{};
 
 }  // namespace msd
 
@@ -71,7 +84,7 @@ using namespace msd;
 
 extern "C" {
 
-int msd_version(void) { return 100; }
+int msd_version(void) { return 200; }
 
 const char *msd_error_string(int code) {
     if (code == MSD_OK) return "ok";
@@ -82,6 +95,18 @@ const char *msd_error_string(int code) {
 int msd_init(void *stream) {
     GnScratch sc;
     return (int)get_scratch(static_cast<hipStream_t>(stream), &sc);
+}
+
+int msd_release(void *stream) {
+    int device = 0;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess) return (int)err;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    auto it = g_scratch.find(ScratchKey{device, static_cast<hipStream_t>(stream)});
+    if (it == g_scratch.end()) return MSD_OK;
+    err = hipFree(it->second.slot_mean);
+    g_scratch.erase(it);
+    return (int)err;
 }
 
 int msd_shutdown(void) {
@@ -99,24 +124,36 @@ int msd_shutdown(void) {
     return rc;
 }
 
-int msd_status(void *stream) {
+int msd_status(void *stream) { return (int)hipStreamSynchronize(static_cast<hipStream_t>(stream)); }
+
+int msd_gn_fallbacks(void *stream, unsigned int *count, int reset) {
+    if (!count) return MSD_ERR_INVALID_VALUE;
+    *count = 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t err = hipStreamSynchronize(s);
     if (err != hipSuccess) return (int)err;
     int device = 0;
     err = hipGetDevice(&device);
     if (err != hipSuccess) return (int)err;
-    GnScratch sc;
+    uint32_t *counters[2] = {nullptr, nullptr};
     {
         std::lock_guard<std::mutex> lock(g_scratch_mutex);
         auto it = g_scratch.find(ScratchKey{device, s});
-        if (it == g_scratch.end()) return MSD_OK;
-        sc = it->second;
+        if (it != g_scratch.end()) counters[0] = it->second.fallbacks;
     }
-    uint32_t flags = 0;
-    err = hipMemcpy(&flags, sc.status, sizeof(flags), hipMemcpyDeviceToHost);
-    if (err != hipSuccess) return (int)err;
-    return flags ? (int)hipErrorLaunchFailure : MSD_OK;
+    for (uint32_t *c : counters) {
+        if (!c) continue;
+        uint32_t v = 0;
+        err = hipMemcpy(&v, c, sizeof(v), hipMemcpyDeviceToHost);
+        if (err != hipSuccess) return (int)err;
+        *count += v;
+        if (reset && v) {
+            v = 0;
+            err = hipMemcpy(c, &v, sizeof(v), hipMemcpyHostToDevice);
+            if (err != hipSuccess) return (int)err;
+        }
+    }
+    return MSD_OK;
 }
 
 int msd_set_tuning(int knob, int value) {
@@ -150,6 +187,9 @@ int msd_set_tuning(int knob, int value) {
             if (value && value != 16 && value != 32 && value != 64) return MSD_ERR_INVALID_VALUE;
             g_tuning.softmax_rows = value;
             return MSD_OK;
+        case MSD_TUNE_GN_SPIN_LIMIT:
+            g_tuning.gn_spin_limit = value;
+            return MSD_OK;
         default:
             return MSD_ERR_INVALID_VALUE;
     }
@@ -157,23 +197,23 @@ int msd_set_tuning(int knob, int value) {
 
 static int groupnorm_entry(const void *x, const void *chunk, void *y, const float *gamma,
                            const float *beta, size_t batch, size_t channels, size_t hw, size_t groups,
-                           float eps, int fuse_silu, int dtype, void *stream) {
+                           float eps, int fuse_silu, int dtype, const GnScratch *fixed, void *stream) {
     if (groups == 0 || channels == 0 || channels % groups != 0) return MSD_ERR_INVALID_VALUE;
     if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
     if (batch * hw != 0 && (!x || !y || !gamma || !beta)) return MSD_ERR_INVALID_VALUE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == MSD_DTYPE_F32)
         return gn_dispatch<float>(x, chunk, y, gamma, beta, batch, channels, hw, groups, eps,
-                                  fuse_silu != 0, s);
+                                  fuse_silu != 0, fixed, s);
     return gn_dispatch<__half>(x, chunk, y, gamma, beta, batch, channels, hw, groups, eps,
-                               fuse_silu != 0, s);
+                               fuse_silu != 0, fixed, s);
 }
 
 int msd_groupnorm(const void *x, void *y, const float *gamma, const float *beta, size_t batch,
                   size_t channels, size_t hw, size_t groups, float eps, int fuse_silu, int dtype,
                   void *stream) {
     return groupnorm_entry(x, nullptr, y, gamma, beta, batch, channels, hw, groups, eps, fuse_silu,
-                           dtype, stream);
+                           dtype, nullptr, stream);
 }
 
 int msd_chunk_add_groupnorm(const void *x, const void *chunk, void *y, const float *gamma,
@@ -181,7 +221,7 @@ int msd_chunk_add_groupnorm(const void *x, const void *chunk, void *y, const flo
                             size_t groups, float eps, int fuse_silu, int dtype, void *stream) {
     if (batch * hw != 0 && !chunk) return MSD_ERR_INVALID_VALUE;
     return groupnorm_entry(x, chunk, y, gamma, beta, batch, channels, hw, groups, eps, fuse_silu,
-                           dtype, stream);
+                           dtype, nullptr, stream);
 }
 
 int msd_groupnorm_tokens(const void *x, void *y, const float *gamma, const float *beta, size_t batch,
@@ -240,6 +280,12 @@ int msd_chunkwise_add(const void *a, const void *chunk, void *c, size_t n, size_
 int msd_geglu(const void *proj, void *out, size_t rows, size_t inner, int dtype, void *stream) {
     if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
     if (rows * inner != 0 && (!proj || !out)) return MSD_ERR_INVALID_VALUE;
+    {   // rows of proj and out have different strides: an overlapping out would be read after it was written
+        const size_t elt = dtype == MSD_DTYPE_F32 ? 4 : 2;
+        const uintptr_t p0 = reinterpret_cast<uintptr_t>(proj), o0 = reinterpret_cast<uintptr_t>(out);
+        const uintptr_t p1 = p0 + rows * 2 * inner * elt, o1 = o0 + rows * inner * elt;
+        if (rows * inner != 0 && o0 < p1 && p0 < o1) return MSD_ERR_INVALID_VALUE;
+    }
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == MSD_DTYPE_F32) return geglu_dispatch<float>(proj, out, rows, inner, s);
     return geglu_dispatch<__half>(proj, out, rows, inner, s);

@@ -459,8 +459,9 @@ int softmax_dispatch(const void *xv, void *yv, size_t rows, size_t cols, int sta
     // The flat kernel pays two LDS round trips per row; it wins once the launch is large
     // enough for the row-per-wavefront kernel to be bound by its 2-byte accesses
     // (measured crossover near 20000 rows of 77).  A set knob forces it for any size.
-    const uint32_t rb = g_tuning.softmax_rows ? (uint32_t)g_tuning.softmax_rows : 64u;
-    const bool flat_pays = g_tuning.softmax_rows ? rows >= rb : rows >= 24576;
+    const int tune_rows = g_tuning.softmax_rows.load(std::memory_order_relaxed);
+    const uint32_t rb = tune_rows ? (uint32_t)tune_rows : 64u;
+    const bool flat_pays = tune_rows ? rows >= rb : rows >= 24576;
     if (cols <= kSmFlatMaxCols && cols >= 8 && flat_pays && aligned16(x) && aligned16(y)) {
         // whole blocks of rb rows through the flat kernel, the rest (if any) row by row below
         const uint32_t blocks = r / rb;

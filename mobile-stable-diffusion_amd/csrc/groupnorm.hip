@@ -15,8 +15,13 @@
 //      works.  All traffic is relaxed agent-scope atomics: no cache flushes.
 //   4. y = fma(x - mean, rstd * gamma[c], beta[c]), optional SiLU, packed store.
 //
-// Workgroups of one unit have adjacent block ids, so every workgroup a waiter
-// depends on is dispatched no later than the waiter; waits are also bounded.
+// Workgroups of one unit have adjacent block ids, so a waiter's siblings are
+// normally dispatched together with it.  Nothing depends on that: a wait is
+// bounded (about a millisecond of polls), and a slice whose sibling has not
+// published by then computes that sibling's statistics itself from the
+// sibling's part of the input, which no workgroup overwrites before it has
+// seen every word of its unit.  The output is the same either way; a counter
+// in the scratch records how often it happened.
 #include "msd_device.h"
 #include "msd_internal.h"
 
@@ -26,7 +31,7 @@ namespace {
 
 constexpr int kGnMaxThreads = 1024;
 constexpr int kGnMaxK = 16;
-constexpr uint32_t kGnSpinLimit = 1u << 22;
+constexpr uint32_t kGnSpinLimit = 2048;  // default poll limit: about half a microsecond per poll
 constexpr int kGenericThreads = 256;
 
 struct GnParams {
@@ -39,6 +44,7 @@ struct GnParams {
     FastDiv hw_vec;          // vectors per channel
     float eps;
     float inv_count;         // 1 / elements per unit
+    uint32_t spin_limit;     // polls before a slice stops waiting for a sibling's words
 };
 
 // Sum over the workgroup (blockDim.x / 64 wavefronts); one barrier.
@@ -60,10 +66,13 @@ __device__ __forceinline__ unsigned long long tagged(uint32_t tag, float v) {
 // (mean, M2); `epoch` is the unit's launch count as lane 0 read it at kernel start.  On return
 // stats[0] = mean and stats[1] = 1/sqrt(var + eps) of the whole unit, in LDS, after a barrier.
 // Slice l covers vectors [l * vec_per_slice, min(vec_per_unit, (l + 1) * vec_per_slice)).
-template <int EPV>
+// `read(l, i)` returns vector i of slice l as the statistics see it (after the optional addend);
+// it is only used when slice l has not published within the poll limit.
+template <typename T, typename Reader>
 __device__ __forceinline__ void gn_exchange(const GnScratch &scratch, const GnParams &p, uint32_t unit,
                                             uint32_t slice, uint32_t epoch, float slice_mean,
-                                            float slice_m2, float *stats) {
+                                            float slice_m2, float *stats, Reader read) {
+    constexpr int EPV = Store<T>::EPV;
     const uint32_t tid = threadIdx.x;
     unsigned long long *slot_mean = scratch.slot_mean + (size_t)unit * kGnMaxSplit;
     unsigned long long *slot_m2 = scratch.slot_m2 + (size_t)unit * kGnMaxSplit;
@@ -77,23 +86,65 @@ __device__ __forceinline__ void gn_exchange(const GnScratch &scratch, const GnPa
         }
         // lane l waits for slice l
         float m_l = 0.0f, q_l = 0.0f, n_l = 0.0f;
+        bool ok = true;
         if (tid < p.split) {
             unsigned long long wm, wq;
             uint32_t polls = 0;
-            bool ok;
             do {
                 wm = __hip_atomic_load(slot_mean + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 wq = __hip_atomic_load(slot_m2 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 ok = (uint32_t)(wm >> 32) == tag && (uint32_t)(wq >> 32) == tag;
                 if (!ok) __builtin_amdgcn_s_sleep(1);
-            } while (!ok && ++polls < kGnSpinLimit);
-            if (!ok)
-                __hip_atomic_fetch_or(scratch.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            } while (!ok && ++polls < p.spin_limit);
             m_l = __uint_as_float((uint32_t)wm);
             q_l = __uint_as_float((uint32_t)wq);
             const uint32_t b = tid * p.vec_per_slice;
             const uint32_t e = min(p.vec_per_unit, b + p.vec_per_slice);
             n_l = (float)((e - b) * EPV);
+        }
+        // Slices that have not published (not dispatched yet, or starved): this wavefront
+        // computes their (mean, M2) from their part of the input, two passes.  A slice stores
+        // output only after it has seen every word of its unit, this slice's included, so what
+        // is read here is still input unless the sibling published in the meantime - then its
+        // words are there when they are read again after the passes, and they win.
+        unsigned long long missing = __builtin_amdgcn_ballot_w64(!ok);
+        if (missing != 0) {  // uniform over the wavefront
+            while (missing != 0) {
+                const uint32_t s = (uint32_t)__builtin_ctzll(missing);
+                missing &= missing - 1;
+                const uint32_t b = s * p.vec_per_slice;
+                const uint32_t n = min(p.vec_per_unit, b + p.vec_per_slice) - b;
+                float sum = 0.0f;
+                for (uint32_t i = tid; i < n; i += kWave) {
+                    float f[EPV];
+                    Store<T>::unpack(read(s, i), f);
+#pragma unroll
+                    for (int e = 0; e < EPV; e++) sum += f[e];
+                }
+                const float mean_s = wave_sum(sum) / (float)(n * EPV);
+                float q = 0.0f;
+                for (uint32_t i = tid; i < n; i += kWave) {
+                    float f[EPV];
+                    Store<T>::unpack(read(s, i), f);
+#pragma unroll
+                    for (int e = 0; e < EPV; e++) {
+                        const float d = f[e] - mean_s;
+                        q = fmaf(d, d, q);
+                    }
+                }
+                const float m2_s = wave_sum(q);
+                if (tid == s) {
+                    const unsigned long long wm =
+                        __hip_atomic_load(slot_mean + s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    const unsigned long long wq =
+                        __hip_atomic_load(slot_m2 + s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    const bool late = (uint32_t)(wm >> 32) == tag && (uint32_t)(wq >> 32) == tag;
+                    m_l = late ? __uint_as_float((uint32_t)wm) : mean_s;
+                    q_l = late ? __uint_as_float((uint32_t)wq) : m2_s;
+                }
+            }
+            if (tid == 0)
+                __hip_atomic_fetch_add(scratch.fallbacks, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         // Chan: mean = sum n_l mean_l / n ; M2 = sum M2_l + sum n_l (mean_l - mean)^2
         const float total_mean = wave_sum(m_l * n_l) * p.inv_count;
@@ -251,7 +302,22 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
         mean = slice_mean;
         rstd = __builtin_amdgcn_rsqf(slice_m2 * p.inv_count + p.eps);
     } else {
-        gn_exchange<EPV>(scratch, p, unit, slice, epoch, slice_mean, slice_m2, stats);
+        // vector i of slice l as the statistics see it (input plus the optional addend)
+        auto read = [&](uint32_t l, uint32_t i) {
+            const uint32_t v = l * p.vec_per_slice + i;
+            u32x4 r = xin[v];
+            if (chunk != nullptr) {
+                const T *cb = chunk + (size_t)(unit / p.groups) * (p.groups * p.ch_per_group);
+                const float cv = Store<T>::load1(cb + ch0 + fast_div(v, p.hw_vec));
+                float f[EPV];
+                Store<T>::unpack(r, f);
+#pragma unroll
+                for (int e = 0; e < EPV; e++) f[e] += cv;
+                r = Store<T>::pack(f);
+            }
+            return r;
+        };
+        gn_exchange<T>(scratch, p, unit, slice, epoch, slice_mean, slice_m2, stats, read);
         mean = stats[0];
         rstd = stats[1];
     }
@@ -406,7 +472,12 @@ __global__ __launch_bounds__(kGnMaxThreads) void gn_tokens_kernel(
         mean = slice_mean;
         rstd = __builtin_amdgcn_rsqf(slice_m2 * p.inv_count + p.eps);
     } else {
-        gn_exchange<EPV>(scratch, p, unit, slice, epoch, slice_mean, slice_m2, stats);
+        // vector i of slice l: channel i / pos_vecs of the group, position vector i % pos_vecs
+        auto read = [&](uint32_t l, uint32_t i) {
+            const uint32_t c = fast_div(i, q.pos_vecs);
+            return xin[(size_t)c * p.hw_vec.d + l * pvs + (i - c * pvs)];
+        };
+        gn_exchange<T>(scratch, p, unit, slice, epoch, slice_mean, slice_m2, stats, read);
         mean = stats[0];
         rstd = stats[1];
     }
@@ -542,8 +613,11 @@ int gn_generic(bool silu, const T *x, const T *chunk, T *y, const float *gamma, 
 template <typename T>
 int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma, const float *beta,
                 size_t batch, size_t channels, size_t hw, size_t groups, float eps, bool silu,
-                hipStream_t stream) {
+                const GnScratch *fixed, hipStream_t stream) {
     constexpr int EPV = Store<T>::EPV;
+    const int tune_split = g_tuning.gn_split.load(std::memory_order_relaxed);
+    const int tune_threads = g_tuning.gn_threads.load(std::memory_order_relaxed);
+    const int tune_spin = g_tuning.gn_spin_limit.load(std::memory_order_relaxed);
     const T *x = static_cast<const T *>(xv);
     const T *chunk = static_cast<const T *>(chunkv);
     T *y = static_cast<T *>(yv);
@@ -552,6 +626,7 @@ int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma
     const size_t units = batch * groups;
     if (units == 0 || unit_size == 0) return MSD_OK;
     if (units > 0x7FFFFFFFull || unit_size > 0x7FFFFFFFull) return MSD_ERR_INVALID_VALUE;
+    if (fixed != nullptr && units > fixed->units) return MSD_ERR_INVALID_VALUE;
     if (!(aligned16(x) && aligned16(y) && hw % EPV == 0))
         return gn_generic<T>(silu, x, chunk, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
 
@@ -562,11 +637,11 @@ int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma
     // smallest power-of-two split whose slices fit in registers
     uint32_t split = 1;
     while ((size_t)split * slice_cap < vec_per_unit && split <= kGnMaxSplit) split *= 2;
-    const bool can_split = units <= kGnMaxUnits;
+    const bool can_split = units <= (fixed != nullptr ? fixed->units : kGnMaxUnits);
     if (split > kGnMaxSplit || (split > 1 && !can_split))
         return gn_generic<T>(silu, x, chunk, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
-    if (g_tuning.gn_split > 0) {
-        uint32_t forced = (uint32_t)g_tuning.gn_split;
+    if (tune_split > 0) {
+        uint32_t forced = (uint32_t)tune_split;
         if (forced > split && can_split && (forced & (forced - 1)) == 0 && forced <= kGnMaxSplit &&
             vec_per_unit >= (size_t)forced * kWave)
             split = forced;
@@ -599,21 +674,23 @@ int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma
     p.hw_vec = make_fast_div((uint32_t)(hw / EPV));
     p.eps = eps;
     p.inv_count = 1.0f / (float)unit_size;
+    p.spin_limit = tune_spin > 0 ? (uint32_t)tune_spin : kGnSpinLimit;
     // every slice must own at least one vector (ceil division can starve the last ones)
     if ((size_t)p.vec_per_slice * (split - 1) >= vec_per_unit)
         return gn_generic<T>(silu, x, chunk, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
 
     uint32_t force_threads = 0;
-    if (g_tuning.gn_threads >= kWave && g_tuning.gn_threads <= kGnMaxThreads &&
-        g_tuning.gn_threads % kWave == 0 &&
-        (size_t)g_tuning.gn_threads * kMaxK >= p.vec_per_slice)
-        force_threads = (uint32_t)g_tuning.gn_threads;
+    if (tune_threads >= kWave && tune_threads <= kGnMaxThreads && tune_threads % kWave == 0 &&
+        (size_t)tune_threads * kMaxK >= p.vec_per_slice)
+        force_threads = (uint32_t)tune_threads;
     const GnPlan pl = plan_slice(p.vec_per_slice, split, force_threads, kMaxK);
     if (pl.k == 0)
         return gn_generic<T>(silu, x, chunk, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
 
-    GnScratch sc{nullptr, nullptr, nullptr, nullptr, nullptr};
-    if (split > 1) {
+    GnScratch sc{nullptr, nullptr, nullptr, nullptr, nullptr, 0};
+    if (fixed != nullptr) {
+        sc = *fixed;
+    } else if (split > 1) {
         const hipError_t err = get_scratch(stream, &sc);
         if (err != hipSuccess) return (int)err;
     }
@@ -634,9 +711,9 @@ int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma
 }
 
 template int gn_dispatch<float>(const void *, const void *, void *, const float *, const float *,
-                                size_t, size_t, size_t, size_t, float, bool, hipStream_t);
+                                size_t, size_t, size_t, size_t, float, bool, const GnScratch *, hipStream_t);
 template int gn_dispatch<__half>(const void *, const void *, void *, const float *, const float *,
-                                 size_t, size_t, size_t, size_t, float, bool, hipStream_t);
+                                 size_t, size_t, size_t, size_t, float, bool, const GnScratch *, hipStream_t);
 
 namespace {
 
@@ -681,7 +758,9 @@ int gn_tokens_dispatch(const void *xv, void *yv, const float *gamma, const float
         want = units >= 256 ? 1 : units >= 128 ? 2 : 4;
         if (units * 4 < 192 && unit_size >= 65536) want = 8;
     }
-    if (g_tuning.gn_split > 0) want = (uint32_t)g_tuning.gn_split;
+    const int tune_split = g_tuning.gn_split.load(std::memory_order_relaxed);
+    const int tune_spin = g_tuning.gn_spin_limit.load(std::memory_order_relaxed);
+    if (tune_split > 0) want = (uint32_t)tune_split;
     uint32_t split = 0;
     for (uint32_t s = 1; s <= kGnMaxSplit; s *= 2) {
         if (hw_vec % s != 0) break;
@@ -705,6 +784,7 @@ int gn_tokens_dispatch(const void *xv, void *yv, const float *gamma, const float
     q.base.hw_vec = make_fast_div((uint32_t)hw_vec);
     q.base.eps = eps;
     q.base.inv_count = 1.0f / (float)unit_size;
+    q.base.spin_limit = tune_spin > 0 ? (uint32_t)tune_spin : kGnSpinLimit;
     q.pos_vecs = make_fast_div((uint32_t)pvs);
     q.row_dwords = make_fast_div((uint32_t)(cpg * sizeof(T) / 4));
     q.hw = (uint32_t)hw;
@@ -714,7 +794,7 @@ int gn_tokens_dispatch(const void *xv, void *yv, const float *gamma, const float
     const size_t lds_bytes = cpg * q.pitch * sizeof(T);
     const GnPlan pl = plan_slice((uint32_t)nvec, split, 0, kMaxK);
     if (pl.k == 0) return generic();
-    GnScratch sc{nullptr, nullptr, nullptr, nullptr, nullptr};
+    GnScratch sc{nullptr, nullptr, nullptr, nullptr, nullptr, 0};
     if (split > 1) {
         const hipError_t err = get_scratch(stream, &sc);
         if (err != hipSuccess) return (int)err;

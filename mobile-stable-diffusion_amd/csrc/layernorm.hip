@@ -195,7 +195,8 @@ void ln_launch(const T *x, const T *res, T *sum, T *y, const float *gamma, const
     // one wavefront per workgroup is 2 - 8 % faster while the launch is small (measured below
     // about 1000 wavefronts); large launches dispatch sooner as 4-wavefront workgroups
     const uint32_t wavefronts = (rows + (kWave / TL) - 1) / (kWave / TL);
-    const uint32_t threads = g_tuning.ln_threads ? (uint32_t)g_tuning.ln_threads
+    const int tune_threads = g_tuning.ln_threads.load(std::memory_order_relaxed);
+    const uint32_t threads = tune_threads ? (uint32_t)tune_threads
                                                  : (wavefronts >= 1024 ? 256u : (uint32_t)kLnThreads);
     const uint32_t rows_per_block = (kWave / TL) * (threads / kWave);
     const uint32_t blocks = (rows + rows_per_block - 1) / rows_per_block;
@@ -271,8 +272,9 @@ int ln_dispatch(const void *xv, const void *resv, void *sumv, void *yv, const fl
             const size_t waves16 = (rows + kWave / tl - 1) / (kWave / tl);
             if (waves16 >= 1024) prefer8 = false;
         }
-        if (g_tuning.ln_chunk == 8) prefer8 = true;
-        if (g_tuning.ln_chunk == 16) prefer8 = false;
+        const int tune_chunk = g_tuning.ln_chunk.load(std::memory_order_relaxed);
+        if (tune_chunk == 8) prefer8 = true;
+        if (tune_chunk == 16) prefer8 = false;
         if (prefer8) done = ln_try<T, 2>(x, res, sum, y, gamma, beta, r, d, eps, inv_dim, stream);
         if (!done) done = ln_try<T, 4>(x, res, sum, y, gamma, beta, r, d, eps, inv_dim, stream);
         if (!done && !prefer8) done = ln_try<T, 2>(x, res, sum, y, gamma, beta, r, d, eps, inv_dim, stream);

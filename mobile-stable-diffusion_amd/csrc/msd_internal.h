@@ -2,6 +2,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <stddef.h>
 #include <stdint.h>
 
@@ -21,29 +22,33 @@ struct GnScratch {
     unsigned long long *slot_m2;    // [kGnMaxUnits][kGnMaxSplit]
     uint32_t *epoch;                // [kGnMaxUnits] launches completed on this unit
     uint32_t *done;                 // [kGnMaxUnits] slices finished in the running launch
-    uint32_t *status;               // [1] sticky: bit 0 = a wait ran out of polls
+    uint32_t *fallbacks;            // [1] slices that stopped waiting and computed a sibling's statistics themselves
+    uint32_t units;                 // units the arrays above have room for
 };
 
 // Per-(device, stream) scratch, created on first use (hipMalloc + hipMemset).
 hipError_t get_scratch(hipStream_t stream, GnScratch *out);
 
-// Tuning overrides set through msd_set_tuning (0 = choose automatically).
+// Tuning overrides set through msd_set_tuning (0 = choose automatically).  Atomics: a launch
+// on one thread may read them while another thread sets them; each launch reads a knob once.
 struct Tuning {
-    int gn_split;
-    int gn_threads;
-    int ln_chunk;
-    int ln_threads;
-    int geglu_vectors;
-    int act_vectors;
-    int softmax_rows;
+    std::atomic<int> gn_split{0};
+    std::atomic<int> gn_threads{0};
+    std::atomic<int> ln_chunk{0};
+    std::atomic<int> ln_threads{0};
+    std::atomic<int> geglu_vectors{0};
+    std::atomic<int> act_vectors{0};
+    std::atomic<int> softmax_rows{0};
+    std::atomic<int> gn_spin_limit{0};
 };
 extern Tuning g_tuning;
 
 // ---- per-dtype dispatchers (T = float or __half), defined in the kernel files ----
+// fixed: scratch to use instead of the stream's own (units beyond its capacity are refused)
 template <typename T>
 int gn_dispatch(const void *x, const void *chunk, void *y, const float *gamma, const float *beta,
                 size_t batch, size_t channels, size_t hw, size_t groups, float eps, bool silu,
-                hipStream_t stream);
+                const GnScratch *fixed, hipStream_t stream);
 // y is token-major [batch, hw, channels]; must not overlap x
 template <typename T>
 int gn_tokens_dispatch(const void *x, void *y, const float *gamma, const float *beta, size_t batch,

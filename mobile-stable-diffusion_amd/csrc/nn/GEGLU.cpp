@@ -20,6 +20,12 @@ int GEGLU::forward(const DeviceBuffer &projected, DeviceBuffer &output, unsigned
                    const hipEvent_t *event_wait_list, hipEvent_t event) {
     checkInput(projected.bytes(), output.bytes(), projected.dtype());
     if (output.dtype() != projected.dtype()) throw std::runtime_error("output type != input type");
+    {   // the kernel reads proj rows and writes out rows of another stride: they must not overlap
+        const char *p0 = static_cast<const char *>(projected.ptr());
+        const char *o0 = static_cast<const char *>(output.ptr());
+        if (projected.bytes() != 0 && o0 < p0 + projected.bytes() && p0 < o0 + output.bytes())
+            throw std::runtime_error("GEGLU not support input overlapping output");
+    }
     for (unsigned i = 0; i < num_events_in_list; i++) {
         const hipError_t err = hipStreamWaitEvent(stream, event_wait_list[i], 0);
         if (err != hipSuccess) return (int)err;

@@ -52,8 +52,8 @@ std::vector<float> normals(Rng &rng, size_t n, float mean, float sigma) {
 
 }  // namespace
 
-UNetNormActStep::UNetNormActStep(hipStream_t stream, size_t batch, DType dtype, unsigned seed)
-    : stream(stream), batch(batch), dtype(dtype) {
+UNetNormActStep::UNetNormActStep(hipStream_t stream, size_t batch, DType dtype, unsigned seed, bool keep_inputs)
+    : keep_inputs(keep_inputs), stream(stream), batch(batch), dtype(dtype) {
     Rng rng{seed};
     const size_t elt = dtype_size(dtype);
     auto activation = [&](size_t n, float sigma) {
@@ -64,19 +64,29 @@ UNetNormActStep::UNetNormActStep(hipStream_t stream, size_t batch, DType dtype, 
         buffers.push_back(DeviceBuffer::allocate(n * elt, dtype));
         return buffers.size() - 1;
     };
+    // a device copy of an input that its layer overwrites, when asked for
+    auto keep = [&](size_t in) -> size_t {
+        if (!keep_inputs) return npos;
+        kept_inputs.push_back(DeviceBuffer::allocate(buffers[in].bytes(), dtype));
+        if (hipMemcpyAsync(kept_inputs.back().ptr(), buffers[in].ptr(), buffers[in].bytes(),
+                           hipMemcpyDeviceToDevice, stream) != hipSuccess)
+            throw std::runtime_error("UNetNormActStep: copy failed");
+        return kept_inputs.size() - 1;
+    };
     auto add_group_norm = [&](size_t channels, size_t hw, bool in_place) {
         group_norms.emplace_back(new GroupNorm(stream, 32, channels, 1e-5f, "", "", batch, true));
-        group_norms.back()->init(normals(rng, channels, 1.0f, 0.1f), normals(rng, channels, 0.0f, 0.1f));
+        std::vector<float> g = normals(rng, channels, 1.0f, 0.1f), b = normals(rng, channels, 0.0f, 0.1f);
+        group_norms.back()->init(g, b);
         const size_t n = batch * channels * hw;
         const size_t in = activation(n, 2.0f);
         const size_t out = in_place ? in : blank(n);
-        ops.push_back({0, group_norms.size() - 1, in, out});
+        ops.push_back({0, group_norms.size() - 1, in, out, {channels, hw}, g, b, in_place ? keep(in) : npos});
         algorithmic_bytes += 2 * n * elt;
     };
     auto add_silu_emb = [&]() {  // SiLU on the [batch, 4*MODEL_CHANNELS] time embedding
         const size_t n = batch * 1280;
         const size_t in = activation(n, 1.0f);
-        ops.push_back({3, 0, in, blank(n)});
+        ops.push_back({3, 0, in, blank(n), {n, 0}, {}, {}, npos});
     };
 
     timestep_dev = DeviceBuffer::allocate(batch * sizeof(int64_t), DType::F32);
@@ -84,7 +94,7 @@ UNetNormActStep::UNetNormActStep(hipStream_t stream, size_t batch, DType dtype, 
     {
         const size_t n = batch * 1280;  // SiLU inside the time-embedding MLP, in place
         const size_t in = activation(n, 1.0f);
-        ops.push_back({3, 0, in, in});
+        ops.push_back({3, 0, in, in, {n, 0}, {}, {}, keep(in)});
     }
     for (const Res &r : kResBlocks) {
         const size_t hw = r.side * r.side;
@@ -95,14 +105,15 @@ UNetNormActStep::UNetNormActStep(hipStream_t stream, size_t batch, DType dtype, 
             const size_t dim = r.cout, rows = batch * hw;
             for (int i = 0; i < 3; i++) {
                 layer_norms.emplace_back(new LayerNorm(stream, dim, "", ""));
-                layer_norms.back()->init(normals(rng, dim, 1.0f, 0.1f), normals(rng, dim, 0.0f, 0.1f));
+                std::vector<float> g = normals(rng, dim, 1.0f, 0.1f), b = normals(rng, dim, 0.0f, 0.1f);
+                layer_norms.back()->init(g, b);
                 const size_t in = activation(rows * dim, 1.0f);
-                ops.push_back({1, layer_norms.size() - 1, in, blank(rows * dim)});
+                ops.push_back({1, layer_norms.size() - 1, in, blank(rows * dim), {rows, dim}, g, b, npos});
                 algorithmic_bytes += 2 * rows * dim * elt;
             }
             geglus.emplace_back(new GEGLU(stream, dim, 4 * dim));
             const size_t in = activation(rows * 8 * dim, 1.0f);
-            ops.push_back({2, geglus.size() - 1, in, blank(rows * 4 * dim)});
+            ops.push_back({2, geglus.size() - 1, in, blank(rows * 4 * dim), {rows, 4 * dim}, {}, {}, npos});
             algorithmic_bytes += 3 * rows * 4 * dim * elt;
         }
     }
@@ -115,11 +126,39 @@ UNetNormActStep::~UNetNormActStep() {
     if (graph) (void)hipGraphDestroy(graph);
 }
 
-int UNetNormActStep::forward(const std::vector<long> &timesteps) {
+void UNetNormActStep::setTimesteps(const std::vector<long> &timesteps) {
     if (timesteps.size() != batch) throw std::runtime_error("one timestep per sample expected");
     std::vector<int64_t> host(timesteps.begin(), timesteps.end());
-    hipError_t err = hipMemcpy(timestep_dev.ptr(), host.data(), batch * sizeof(int64_t), hipMemcpyHostToDevice);
-    if (err != hipSuccess) return (int)err;
+    // ordered behind the work already on the stream (an earlier step may still read the old values)
+    hipError_t err = hipStreamSynchronize(stream);
+    if (err == hipSuccess)
+        err = hipMemcpy(timestep_dev.ptr(), host.data(), batch * sizeof(int64_t), hipMemcpyHostToDevice);
+    if (err != hipSuccess)
+        throw std::runtime_error(std::string("UNetNormActStep: timestep upload failed: ") + hipGetErrorString(err));
+}
+
+int UNetNormActStep::restoreInputs() {
+    if (!keep_inputs) throw std::runtime_error("UNetNormActStep was built without keep_inputs");
+    for (const Op &op : ops) {
+        if (op.kept == npos) continue;
+        const hipError_t err = hipMemcpyAsync(buffers[op.in].ptr(), kept_inputs[op.kept].ptr(),
+                                              buffers[op.in].bytes(), hipMemcpyDeviceToDevice, stream);
+        if (err != hipSuccess) return (int)err;
+    }
+    return MSD_OK;
+}
+
+UNetNormActStep::OpInfo UNetNormActStep::opInfo(size_t i) const {
+    const Op &op = ops.at(i);
+    return OpInfo{op.kind, {op.dims[0], op.dims[1]}, op.in == op.out};
+}
+
+std::vector<float> UNetNormActStep::downloadInput(size_t i) const { return util::download(buffers[ops.at(i).in], stream); }
+std::vector<float> UNetNormActStep::downloadOutput(size_t i) const { return util::download(buffers[ops.at(i).out], stream); }
+std::vector<float> UNetNormActStep::downloadEmbedding() const { return util::download(embedding, stream); }
+
+int UNetNormActStep::forward(const std::vector<long> &timesteps) {
+    setTimesteps(timesteps);
     int rc = msd_timestep_embedding(static_cast<const int64_t *>(timestep_dev.ptr()), embedding.ptr(), batch,
                                     320, 10000.0f, (int)dtype, stream);
     for (size_t i = 0; i < ops.size() && rc == MSD_OK; i++) {
@@ -151,10 +190,14 @@ int UNetNormActStep::forwardGraph() {
             }
         }
         err = hipStreamEndCapture(stream, &graph);
-        if (rc != MSD_OK) return rc;
-        if (err != hipSuccess) return (int)err;
-        err = hipGraphInstantiate(&graph_exec, graph, nullptr, nullptr, 0);
-        if (err != hipSuccess) return (int)err;
+        if (rc == MSD_OK && err == hipSuccess) err = hipGraphInstantiate(&graph_exec, graph, nullptr, nullptr, 0);
+        if (rc != MSD_OK || err != hipSuccess) {  // nothing half-built survives: the next call starts over
+            if (graph_exec) (void)hipGraphExecDestroy(graph_exec);
+            if (graph) (void)hipGraphDestroy(graph);
+            graph_exec = nullptr;
+            graph = nullptr;
+            return rc != MSD_OK ? rc : (int)err;
+        }
     }
     return (int)hipGraphLaunch(graph_exec, stream);
 }

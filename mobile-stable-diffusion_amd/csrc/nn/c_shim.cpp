@@ -287,14 +287,52 @@ int msdnn_test_buffer(void *stream, void *ptr, size_t bytes, int dtype, const ch
 }
 
 // ---- one UNet step of the path
-void *msdnn_step_create(void *stream, size_t batch, int dtype) {
+void *msdnn_step_create(void *stream, size_t batch, int dtype, int keep_inputs) {
     UNetNormActStep *s = nullptr;
     guarded([&] {
         s = new UNetNormActStep(static_cast<hipStream_t>(stream), batch,
-                                dtype == MSD_DTYPE_F16 ? DType::F16 : DType::F32);
+                                dtype == MSD_DTYPE_F16 ? DType::F16 : DType::F32, 5001, keep_inputs != 0);
         return 0;
     });
     return s;
+}
+// what launch i works on: kind 0 GroupNorm+SiLU {channels, hw}, 1 LayerNorm {rows, dim},
+// 2 GEGLU {rows, inner}, 3 SiLU {n, 0}
+size_t msdnn_step_num_ops(void *h) { return static_cast<UNetNormActStep *>(h)->numOps(); }
+int msdnn_step_op_info(void *h, size_t i, int *kind, size_t *dims, int *in_place) {
+    return guarded([&] {
+        const UNetNormActStep::OpInfo info = static_cast<UNetNormActStep *>(h)->opInfo(i);
+        *kind = info.kind;
+        dims[0] = info.dims[0];
+        dims[1] = info.dims[1];
+        *in_place = info.in_place ? 1 : 0;
+        return 0;
+    });
+}
+// which: 0 input of launch i, 1 output of launch i, 2 the timestep embedding (i ignored);
+// writes at most cap floats, *count receives the element count
+int msdnn_step_download(void *h, size_t i, int which, float *dst, size_t cap, size_t *count) {
+    return guarded([&] {
+        UNetNormActStep *s = static_cast<UNetNormActStep *>(h);
+        const std::vector<float> v = which == 0 ? s->downloadInput(i) : which == 1 ? s->downloadOutput(i)
+                                                                                    : s->downloadEmbedding();
+        if (count) *count = v.size();
+        if (dst) memcpy(dst, v.data(), sizeof(float) * (v.size() < cap ? v.size() : cap));
+        return 0;
+    });
+}
+int msdnn_step_affine(void *h, size_t i, float *gamma, float *beta, size_t cap) {
+    return guarded([&] {
+        UNetNormActStep *s = static_cast<UNetNormActStep *>(h);
+        const std::vector<float> &g = s->weight(i), &b = s->bias(i);
+        if (g.size() > cap || b.size() > cap) throw std::runtime_error("msdnn_step_affine: buffer too small");
+        memcpy(gamma, g.data(), sizeof(float) * g.size());
+        memcpy(beta, b.data(), sizeof(float) * b.size());
+        return (int)g.size();
+    });
+}
+int msdnn_step_restore(void *h) {
+    return guarded([&] { return static_cast<UNetNormActStep *>(h)->restoreInputs(); });
 }
 size_t msdnn_step_bytes(void *h) { return static_cast<UNetNormActStep *>(h)->bytesPerStep(); }
 size_t msdnn_step_launches(void *h) { return static_cast<UNetNormActStep *>(h)->launchesPerStep(); }
@@ -304,6 +342,7 @@ int msdnn_step_run(void *h, int steps, int graph, const long *timesteps, size_t 
         UNetNormActStep *s = static_cast<UNetNormActStep *>(h);
         const std::vector<long> t(timesteps, timesteps + batch);
         int rc = 0;
+        if (graph) s->setTimesteps(t);
         for (int i = 0; i < steps && rc == 0; i++) rc = graph ? s->forwardGraph() : s->forward(t);
         return rc;
     });

@@ -71,15 +71,26 @@ Array load(const std::string &path) {
     const size_t open = shape_text.find('('), close = shape_text.find(')');
     if (open != 0 || close == std::string::npos)
         throw std::runtime_error("parse_npy_header: failed to find header keyword: '(' or ')'");
+    // what is left of the file bounds the element count: a header that claims more is refused
+    // before anything is allocated, and the running product cannot overflow below that bound
+    const long data_start = ftell(f.fp);
+    if (data_start < 0 || fseek(f.fp, 0, SEEK_END) != 0) throw std::runtime_error("npy_load: cannot seek in " + path);
+    const long file_end = ftell(f.fp);
+    if (file_end < data_start || fseek(f.fp, data_start, SEEK_SET) != 0)
+        throw std::runtime_error("npy_load: cannot seek in " + path);
+    const size_t max_vals = (size_t)(file_end - data_start) / sizeof(float);
     Array out;
     size_t total = 1;
     size_t i = open + 1;
     while (i < close) {
         if (shape_text[i] >= '0' && shape_text[i] <= '9') {
             size_t v = 0;
-            while (i < close && shape_text[i] >= '0' && shape_text[i] <= '9')
+            while (i < close && shape_text[i] >= '0' && shape_text[i] <= '9') {
+                if (v > max_vals) throw std::runtime_error("nread != num_bytes");  // longer than the file
                 v = v * 10 + (size_t)(shape_text[i++] - '0');
+            }
             out.shape.push_back(v);
+            if (v != 0 && total > max_vals / v) throw std::runtime_error("nread != num_bytes");
             total *= v;
         } else {
             i++;

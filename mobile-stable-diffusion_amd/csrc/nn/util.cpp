@@ -202,6 +202,9 @@ bool debugTiming() {
 
 LaunchTimer::LaunchTimer(hipStream_t stream) : stream_(stream) {
     if (!debugTiming()) return;
+    // no timing inside a stream capture: waiting for an event there would invalidate it
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream_, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) return;
     if (hipEventCreate(&start_) != hipSuccess || hipEventCreate(&stop_) != hipSuccess ||
         hipEventRecord(start_, stream_) != hipSuccess) {
         if (start_) (void)hipEventDestroy(start_);

@@ -238,7 +238,8 @@ int geglu_dispatch(const void *pv, void *ov, size_t rows, size_t inner, hipStrea
         // one vector per lane: these launches are short enough that a lane's dependent ALU chain
         // is on the critical path, and more, lighter wavefronts overlap it with other loads
         // (measured 9 - 30 % faster than 4 vectors per lane at every UNet shape)
-        const int unroll = g_tuning.geglu_vectors ? g_tuning.geglu_vectors : 1;
+        const int tune_vectors = g_tuning.geglu_vectors.load(std::memory_order_relaxed);
+        const int unroll = tune_vectors ? tune_vectors : 1;
         const uint32_t ov = (uint32_t)out_vecs;
         auto blocks = [&](int u) { return (uint32_t)((out_vecs + kGegluThreads * u - 1) / (kGegluThreads * u)); };
         if (unroll == 1)
@@ -266,7 +267,8 @@ int act_launch(const void *xv, void *yv, size_t n, hipStream_t stream) {
     if (n == 0) return MSD_OK;
     const size_t vecs = n / EPV;
     if (aligned16(x) && aligned16(y) && vecs < 0x7FFFFFFFull) {
-        const int unroll = g_tuning.act_vectors ? g_tuning.act_vectors : kStreamUnroll;
+        const int tune_vectors = g_tuning.act_vectors.load(std::memory_order_relaxed);
+        const int unroll = tune_vectors ? tune_vectors : kStreamUnroll;
         const uint32_t blocks = vecs ? stream_blocks(vecs, unroll) : 1u;
         if (unroll == 4)
             hipLaunchKernelGGL((act_kernel<T, OP, 4>), dim3(blocks), dim3(kStreamThreads), 0, stream, x, y,

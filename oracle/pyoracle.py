@@ -32,6 +32,17 @@ def build():
     return LIB_PATH
 
 
+def build_flags():
+    """The compiler flags of liboracle.so as oracle/Makefile states them."""
+    try:
+        for line in open(os.path.join(_DIR, "Makefile")):
+            if line.startswith("CFLAGS"):
+                return "gcc " + line.split(":=", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def lib():
     global _lib
     if _lib is not None:

@@ -14,6 +14,25 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def pytest_sessionfinish(session, exitstatus):
+    # per-label fp16 parity figures of this run (worst error, elements over a bare 2e-3)
+    import json
+    from tolerances import FP16_REPORT
+    if FP16_REPORT:
+        out = os.path.join(REPO, "gpurun_out")
+        os.makedirs(out, exist_ok=True)
+        path = os.path.join(out, "parity_fp16.json")
+        merged = {}
+        try:  # a run of part of the suite keeps the other labels of an earlier run
+            with open(path) as f:
+                merged = json.load(f)
+        except (OSError, ValueError):
+            pass
+        merged.update(FP16_REPORT)
+        with open(path, "w") as f:
+            json.dump(merged, f, indent=1, sort_keys=True)
+
+
 @pytest.fixture(scope="session")
 def msd():
     """The product package (ctypes access to the HIP library); raises if it is not built."""

@@ -73,8 +73,17 @@ def test_argument_validation_needs_no_gpu(msd):
     assert lib.msd_set_tuning(1, 100) == 1    # threads must be a multiple of 64
     assert lib.msd_set_tuning(2, 12) == 1 and lib.msd_set_tuning(4, 3) == 1 and lib.msd_set_tuning(99, 1) == 1
     assert lib.msd_set_tuning(6, 48) == 1     # softmax rows per workgroup: 16, 32 or 64
-    for knob in range(7):
+    for knob in range(8):
         assert lib.msd_set_tuning(knob, 0) == 0
+    # GEGLU rows of input and output have different strides: any overlap is refused
+    # (addresses are never dereferenced: the check comes before the launch)
+    base = 1 << 20
+    rows, inner = 4, 64  # fp16: proj 4 * 128 * 2 = 1024 bytes, out 512 bytes
+    p = ctypes.c_void_p
+    assert lib.msd_geglu(p(base), p(base), rows, inner, 1, None) == 1            # in place
+    assert lib.msd_geglu(p(base), p(base + 1008), rows, inner, 1, None) == 1     # out starts inside proj
+    assert lib.msd_geglu(p(base + 496), p(base), rows, inner, 1, None) == 1      # proj starts inside out
+    assert lib.msd_gn_fallbacks(None, None, 0) == 1
     # the neighbours of the path
     assert lib.msd_linear_rows(None, None, None, None, 9, 4, 8, 0, 0, 0, None) == 1   # more than 8 rows
     assert lib.msd_linear_rows(None, None, None, None, 2, 4, 8, 0, 0, 0, None) == 1   # null pointers

@@ -2,8 +2,8 @@
 
 Same seeded inputs go to the oracle (float32 restatement of the reference's
 kernels) and to the GPU.  fp32 storage: 1e-5 relative; fp16 storage: the oracle
-runs on fp16-rounded inputs and its output is rounded to fp16 (see
-tolerances.py).  Shapes are the reference's SD UNet / text-encoder shapes at
+runs on fp16-rounded inputs and the stored fp16 result must be the correct
+rounding of a value within 1e-5 of its unrounded output (see tolerances.py).  Shapes are the reference's SD UNet / text-encoder shapes at
 batch 2 plus the edge cases the reference's preconditions and the kernels'
 dispatch split on.
 """
@@ -48,7 +48,7 @@ def _run_groupnorm(msd, orc, cuda, x, g, b, groups, eps, silu, half, inplace=Fal
                         out=xd if inplace else None)
     got = out.float().cpu().numpy()
     if half:
-        return assert_close_f16(got, orc.round_to_half(ref), "groupnorm f16 %s" % (x.shape,))
+        return assert_close_f16(got, ref, "groupnorm f16 %s" % (x.shape,))
     return assert_close_f32(got, ref, what="groupnorm f32 %s" % (x.shape,)), None
 
 
@@ -108,6 +108,39 @@ def test_groupnorm_every_split_factor(msd, orc, cuda, split, threads):
     assert msd.status() == 0
 
 
+@pytest.mark.parametrize("split", [2, 4, 16])
+def test_groupnorm_slice_that_stops_waiting_computes_its_siblings_statistics(msd, orc, cuda, split):
+    """With a poll limit of one, nearly every workgroup gives up on its siblings at once and
+    computes their statistics from the input itself (what a starved workgroup does after a
+    millisecond in normal operation).  Every kernel still runs to its normal end and the
+    output must be the usual one, in place too (siblings overwrite their part of the input only
+    after they have seen every word of the unit)."""
+    lib = msd.load_library()
+    x = orc.normal((2, 320, 64, 64), seed=97, sigma=2.0, mean=1.0)
+    g, b = _affine(orc, 320, 97)
+    msd.gn_fallbacks(reset=True)
+    try:
+        assert lib.msd_set_tuning(msd.TUNE_GN_SPLIT, split) == 0
+        assert lib.msd_set_tuning(msd.TUNE_GN_SPIN_LIMIT, 1) == 0
+        for half in (False, True):
+            for inplace in (False, True):
+                _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half, inplace=inplace)
+        # the token-major kernel shares the exchange
+        xin = orc.round_to_half(x[:, :, :32, :32])
+        tok = msd.groupnorm_tokens(_to_dev(xin, cuda, True), _to_dev(g, cuda), _to_dev(b, cuda), 32, 1e-6)
+        ref = orc.groupnorm(xin, g, b, 32, 1e-6, False).reshape(2, 320, -1).transpose(0, 2, 1)
+        assert_close_f16(tok.float().cpu().numpy(), ref, "gn tokens, forced give-up")
+    finally:
+        lib.msd_set_tuning(msd.TUNE_GN_SPLIT, 0)
+        lib.msd_set_tuning(msd.TUNE_GN_SPIN_LIMIT, 0)
+    assert msd.gn_fallbacks() > 0  # the path was really taken
+    # back to the normal limit: no workgroup gives up on an idle GPU
+    msd.gn_fallbacks(reset=True)
+    _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, True)
+    assert msd.gn_fallbacks() == 0
+    assert msd.status() == 0
+
+
 def test_groupnorm_repeated_launches_reuse_scratch(msd, orc, cuda):
     # the arrival counters are never reset: many launches with changing split factors
     lib = msd.load_library()
@@ -141,7 +174,7 @@ def test_groupnorm_edge_shapes(msd, orc, cuda, shape, groups, half):
     xd = _to_dev(xin, cuda, half)                         # reference's % 64 precondition
     got = msd.groupnorm(xd, _to_dev(g, cuda), _to_dev(b, cuda), groups, 1e-5, True).float().cpu().numpy()
     if half:
-        assert_close_f16(got, orc.round_to_half(ref.astype(np.float32)), "gn edge f16")
+        assert_close_f16(got, ref.astype(np.float32), "gn edge f16")
     else:
         assert_close_f32(got, ref, what="gn edge f32")
     assert msd.status() == 0
@@ -212,7 +245,7 @@ def test_groupnorm_golden_fixtures(msd, golden, cuda):
 def test_config3_layernorm_fp16(msd, orc, cuda, rows, dim, seed):
     x = orc.round_to_half(orc.normal((2, rows // 2, dim), seed=seed))
     g, b = _affine(orc, dim, seed)
-    ref = orc.round_to_half(orc.layernorm(x, g, b, 1e-5))
+    ref = orc.layernorm(x, g, b, 1e-5)
     got = msd.layernorm(_to_dev(x, cuda, True), _to_dev(g, cuda), _to_dev(b, cuda)).float().cpu().numpy()
     worst, exact = assert_close_f16(got, ref, "layernorm f16 %dx%d" % (rows, dim))
     assert exact > 0.99
@@ -239,7 +272,7 @@ def test_layernorm_dims_and_ragged_rows(msd, orc, cuda, rows, dim, half):
     ref = orc.layernorm64(xin, g, b, 1e-5)
     got = msd.layernorm(_to_dev(xin, cuda, half), _to_dev(g, cuda), _to_dev(b, cuda)).float().cpu().numpy()
     if half:
-        assert_close_f16(got, orc.round_to_half(ref.astype(np.float32)), "ln dims f16")
+        assert_close_f16(got, ref.astype(np.float32), "ln dims f16")
     else:
         assert_close_f32(got, ref, what="ln dims f32")
 
@@ -258,7 +291,7 @@ def test_layernorm_forced_chunk_width(msd, orc, cuda, chunk, threads):
             ref = orc.layernorm(xin, g, b, 1e-5)
             got = msd.layernorm(_to_dev(xin, cuda, half), _to_dev(g, cuda), _to_dev(b, cuda)).float().cpu().numpy()
             if half:
-                assert_close_f16(got, orc.round_to_half(ref), "ln chunk f16")
+                assert_close_f16(got, ref, "ln chunk f16")
             else:
                 assert_close_f32(got, ref, what="ln chunk f32")
     finally:
@@ -281,7 +314,7 @@ def test_layernorm_in_place_fixtures_and_empty(msd, orc, golden, cuda):
                                              (128, 5120, 3008)])
 def test_config3_geglu_fp16(msd, orc, cuda, rows, inner, seed):
     proj = orc.round_to_half(orc.normal((rows, 2 * inner), seed=seed))
-    ref = orc.round_to_half(orc.geglu(proj))
+    ref = orc.geglu(proj)
     got = msd.geglu(_to_dev(proj, cuda, True)).float().cpu().numpy()
     worst, exact = assert_close_f16(got, ref, "geglu f16 %dx%d" % (rows, inner))
     assert exact > 0.99
@@ -295,7 +328,7 @@ def test_geglu_shapes_fp32_fp16(msd, orc, golden, cuda, rows, inner, half):
     ref = orc.geglu(pin)
     got = msd.geglu(_to_dev(pin, cuda, half)).float().cpu().numpy()
     if half:
-        assert_close_f16(got, orc.round_to_half(ref), "geglu shapes f16")
+        assert_close_f16(got, ref, "geglu shapes f16")
     else:
         assert_close_f32(got, ref, what="geglu shapes f32")
         assert_close_f32(msd.geglu(_to_dev(golden["geglu_proj"], cuda)).cpu().numpy(), golden["geglu_y"])
@@ -312,7 +345,7 @@ def test_geglu_forced_vectors_per_lane(msd, orc, cuda, unroll):
         for rows, inner in [(2048, 2560), (77, 1288), (3, 8), (1000, 24)]:
             proj = orc.round_to_half(orc.normal((rows, 2 * inner), seed=rows + unroll, sigma=1.5))
             got = msd.geglu(_to_dev(proj, cuda, True)).float().cpu().numpy()
-            assert_close_f16(got, orc.round_to_half(orc.geglu(proj)), "geglu unroll")
+            assert_close_f16(got, orc.geglu(proj), "geglu unroll")
     finally:
         lib.msd_set_tuning(msd.TUNE_GEGLU_VECTORS, 0)
         lib.msd_set_tuning(msd.TUNE_ACT_VECTORS, 0)
@@ -331,7 +364,7 @@ def test_activations(msd, orc, golden, cuda, name, half):
         xd = _to_dev(xin, cuda, half)
         got = fn(xd, out=xd).float().cpu().numpy()  # in place, like every reference call site
         if half:
-            assert_close_f16(got, orc.round_to_half(ref_fn(xin)), name + " f16")
+            assert_close_f16(got, ref_fn(xin), name + " f16")
         else:
             assert_close_f32(got, ref_fn(xin), what=name + " f32")
     if not half:
@@ -364,7 +397,7 @@ def test_timestep_embedding_all_timesteps(msd, orc, golden, cuda):
     assert np.abs(g2 - golden["temb_f64"]).max() < 1.3e-4  # |t| * ulp(freq) at t ~ 1000
     # fp16 storage and another dim / period
     h = msd.timestep_embedding(torch.from_numpy(ts[:64]).to(cuda), 320, dtype=torch.float16).float().cpu().numpy()
-    assert_close_f16(h, orc.round_to_half(ref[:64]), "temb f16")
+    assert_close_f16(h, ref[:64], "temb f16")
     o = msd.timestep_embedding(torch.tensor([13], device=cuda), 64, max_period=100.0).cpu().numpy()[0]
     assert_close_f32(o, orc.timestep_embedding(13, 64, 100.0))
 
@@ -423,8 +456,8 @@ def test_groupnorm_graph_replay_matches_eager(msd, orc, cuda):
         assert msd.status() == 0
     # and the eager result is the right one
     for x0, (g, b), (ey, ez) in zip(xs0, gbs, eager):
-        assert_close_f16(ey.float().cpu().numpy(), orc.round_to_half(orc.groupnorm(x0, g, b, 32, 1e-5, True)), "gn graph")
-        assert_close_f16(ez.float().cpu().numpy(), orc.round_to_half(orc.groupnorm(x0, g, b, 32, 1e-6, False)), "gn graph")
+        assert_close_f16(ey.float().cpu().numpy(), orc.groupnorm(x0, g, b, 32, 1e-5, True), "gn graph")
+        assert_close_f16(ez.float().cpu().numpy(), orc.groupnorm(x0, g, b, 32, 1e-6, False), "gn graph")
 
 
 def test_groupnorm_two_streams_have_private_scratch(msd, orc, cuda):
@@ -445,8 +478,8 @@ def test_groupnorm_two_streams_have_private_scratch(msd, orc, cuda):
         with torch.cuda.stream(s2):
             outs2.append(msd.groupnorm(d2, *a2, 32, 1e-5, True))
     torch.cuda.synchronize()
-    r1 = orc.round_to_half(orc.groupnorm(x1, g1, b1, 32, 1e-5, True))
-    r2 = orc.round_to_half(orc.groupnorm(x2, g2, b2, 32, 1e-5, True))
+    r1 = orc.groupnorm(x1, g1, b1, 32, 1e-5, True)
+    r2 = orc.groupnorm(x2, g2, b2, 32, 1e-5, True)
     for o in outs1:
         assert torch.equal(o, outs1[0])
     for o in outs2:
@@ -485,7 +518,7 @@ def test_groupnorm_many_units_and_register_limits(msd, orc, cuda):
         got = msd.groupnorm(_to_dev(xin, cuda, half), _to_dev(g, cuda), _to_dev(b, cuda), groups, 1e-5, True)
         got = got.float().cpu().numpy()
         if half:
-            assert_close_f16(got, orc.round_to_half(ref.astype(np.float32)), "gn limits f16")
+            assert_close_f16(got, ref.astype(np.float32), "gn limits f16")
         else:
             assert_close_f32(got, ref, what="gn limits f32")
     assert msd.status() == 0
