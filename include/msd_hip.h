@@ -24,6 +24,7 @@ extern "C" {
 
 #define MSD_OK 0
 #define MSD_ERR_INVALID_VALUE 1 /* == hipErrorInvalidValue */
+#define MSD_ERR_SCRATCH_LIMIT (-2) /* msd_groupnorm_noalloc: batch * groups above its fixed scratch */
 
 /* storage type of activations; arithmetic is always float32 */
 #define MSD_DTYPE_F32 0
@@ -43,7 +44,8 @@ const char *msd_error_string(int code);
  * stream capture.  A graph captured on a stream keeps using that stream's
  * scratch: GroupNorm launches that share scratch must not run concurrently
  * (do not replay such a graph on a second stream while the first is busy with
- * GroupNorms).  hipStreamPerThread is refused (one handle, a
+ * GroupNorms).  Also looks up the device address of msd_groupnorm_noalloc's fixed
+ * scratch on the current device.  hipStreamPerThread is refused (one handle, a
  * different stream in every thread).  No reference counterpart (the reference
  * allocates two temporaries per forward, M/nn/GroupNorm.cpp:95-103).
  */
@@ -68,8 +70,8 @@ int msd_status(void *stream);
  * Diagnostic.  Workgroups that share one (sample, group) exchange partial statistics; one
  * that does not receive a sibling's within its poll limit computes them itself from the
  * input, so the output is right either way.  This synchronises `stream` and returns in
- * *count how often that happened so far on the stream's scratch (0 on an idle GPU);
- * reset != 0 clears the counter.
+ * *count how often that happened so far on the stream's scratch and on the fixed scratch of
+ * msd_groupnorm_noalloc (0 on an idle GPU); reset != 0 clears the counters.
  */
 int msd_gn_fallbacks(void *stream, unsigned int *count, int reset);
 
@@ -102,6 +104,21 @@ int msd_set_tuning(int knob, int value);
 int msd_groupnorm(const void *x, void *y, const float *gamma, const float *beta,
                   size_t batch, size_t channels, size_t hw, size_t groups, float eps,
                   int fuse_silu, int dtype, void *stream);
+
+/*
+ * msd_groupnorm for callers that cannot allocate (code under stream capture, tight serving
+ * loops, harnesses that forbid hipMalloc): same arguments, same kernels, same result bit for
+ * bit, but the workgroups' exchange area is a fixed 1 MiB array inside the library's code
+ * object instead of a per-stream allocation, so the call never allocates or frees (its first
+ * call on a device looks the array's address up; msd_init does that ahead of time).  Limit:
+ * batch * groups <= 1024, otherwise MSD_ERR_SCRATCH_LIMIT.  Every stream of a device shares
+ * the one array: calls that overlap in time on one GPU race (their results are undefined);
+ * calls ordered by a stream or by events are fine, and nothing needs clearing between them.
+ * Each GPU holds its array until the process ends.  No counterpart in the reference.
+ */
+int msd_groupnorm_noalloc(const void *x, void *y, const float *gamma, const float *beta,
+                          size_t batch, size_t channels, size_t hw, size_t groups, float eps,
+                          int fuse_silu, int dtype, void *stream);
 
 /*
  * GroupNorm whose result is stored token-major: x is [batch, channels, hw], y is

@@ -19,11 +19,12 @@ DTYPE_F32 = 0
 DTYPE_F16 = 1
 TUNE_GN_SPLIT, TUNE_GN_THREADS, TUNE_LN_CHUNK, TUNE_LN_THREADS, TUNE_GEGLU_VECTORS, TUNE_ACT_VECTORS, \
     TUNE_SOFTMAX_ROWS, TUNE_GN_SPIN_LIMIT = range(8)
+ERR_SCRATCH_LIMIT = -2
 
 # every symbol include/msd_hip.h declares
 C_ABI_SYMBOLS = (
     "msd_version", "msd_error_string", "msd_init", "msd_release", "msd_shutdown", "msd_status",
-    "msd_gn_fallbacks", "msd_set_tuning", "msd_groupnorm", "msd_layernorm", "msd_geglu",
+    "msd_gn_fallbacks", "msd_set_tuning", "msd_groupnorm", "msd_groupnorm_noalloc", "msd_layernorm", "msd_geglu",
     "msd_silu", "msd_gelu", "msd_quick_gelu", "msd_timestep_embedding", "msd_ddim_timesteps",
     "msd_elemwise_add", "msd_chunkwise_add", "msd_chunk_add_groupnorm", "msd_add_layernorm", "msd_copy",
     "msd_groupnorm_tokens", "msd_permute_0_2_1",
@@ -60,6 +61,7 @@ def load_library(path=None):
     lib.msd_gn_fallbacks.argtypes = [vp, ctypes.POINTER(ctypes.c_uint), it]
     lib.msd_set_tuning.argtypes = [it, it]
     lib.msd_groupnorm.argtypes = [vp, vp, vp, vp, sz, sz, sz, sz, fl, it, it, vp]
+    lib.msd_groupnorm_noalloc.argtypes = [vp, vp, vp, vp, sz, sz, sz, sz, fl, it, it, vp]
     lib.msd_layernorm.argtypes = [vp, vp, vp, vp, sz, sz, fl, it, vp]
     lib.msd_geglu.argtypes = [vp, vp, sz, sz, it, vp]
     lib.msd_copy.argtypes = [vp, vp, sz, vp]
@@ -144,13 +146,14 @@ def gn_fallbacks(reset=False):
     return n.value
 
 
-def groupnorm(x, gamma, beta, groups, eps=1e-5, fuse_silu=False, out=None):
-    """x: [batch, C, ...] device tensor; gamma/beta float32 [C]; out may be x (in place)."""
+def groupnorm(x, gamma, beta, groups, eps=1e-5, fuse_silu=False, out=None, noalloc=False):
+    """x: [batch, C, ...] device tensor; gamma/beta float32 [C]; out may be x (in place).
+    noalloc: go through msd_groupnorm_noalloc (fixed scratch, batch * groups <= 1024)."""
     import torch
     out = torch.empty_like(x) if out is None else out
     batch, channels = x.shape[0], x.shape[1]
     hw = x.numel() // (batch * channels) if batch * channels else 0
-    fn = load_library().msd_groupnorm
+    fn = load_library().msd_groupnorm_noalloc if noalloc else load_library().msd_groupnorm
     check(fn(_dev(x), _same(out, x, x.numel(), "out"), _affine(gamma, channels, x, "gamma"),
              _affine(beta, channels, x, "beta"), batch, channels, hw, groups, eps, int(fuse_silu),
              _dtype_code(x), _stream()))

@@ -42,6 +42,16 @@ GnScratch carve(char *base, size_t units) {
     return s;
 }
 
+// Scratch of the entry point that allocates nothing: part of the code object, one copy per
+// device, zero when the module is loaded (tags, launch counts and counters start at zero and
+// are never reset: see groupnorm.hip).  In host code this name is only a handle for
+// hipGetSymbolAddress; kernels get the device address that call returns.
+constexpr uint32_t kStaticUnits = 1024;
+static __device__ __align__(256) unsigned char scratch[scratch_bytes(kStaticUnits)];
+
+constexpr int kMaxDevices = 64;
+char *g_static_base[kMaxDevices] = {nullptr};  // device address of `scratch`, per device
+
 }  // namespace
 
 // Scratch is private to a (device, stream) pair: launches on one stream are ordered, so a
@@ -76,6 +86,24 @@ hipError_t get_scratch(hipStream_t stream, GnScratch *out) {
     return hipSuccess;
 }
 
+// The device address of the static scratch on the current device, looked up once per device.
+hipError_t get_static_scratch(GnScratch *out) {
+    int device = 0;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess) return err;
+    if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_static_base[device] == nullptr) {
+        void *ptr = nullptr;
+        err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (err != hipSuccess) return err;
+        if (ptr == nullptr) return hipErrorInvalidSymbol;
+        g_static_base[device] = static_cast<char *>(ptr);
+    }
+    *out = carve(g_static_base[device], kStaticUnits);
+    return hipSuccess;
+}
+
 Tuning g_tuning{};
 
 }  // namespace msd
@@ -89,11 +117,15 @@ int msd_version(void) { return 200; }
 const char *msd_error_string(int code) {
     if (code == MSD_OK) return "ok";
     if (code == MSD_ERR_INVALID_VALUE) return "invalid value (shape, pointer or dtype rejected)";
+    if (code == MSD_ERR_SCRATCH_LIMIT)
+        return "msd_groupnorm_noalloc: batch * groups exceeds the 1024 units its fixed scratch holds";
     return hipGetErrorString(static_cast<hipError_t>(code));
 }
 
 int msd_init(void *stream) {
     GnScratch sc;
+    hipError_t err = get_static_scratch(&sc);
+    if (err != hipSuccess) return (int)err;
     return (int)get_scratch(static_cast<hipStream_t>(stream), &sc);
 }
 
@@ -140,6 +172,8 @@ int msd_gn_fallbacks(void *stream, unsigned int *count, int reset) {
         std::lock_guard<std::mutex> lock(g_scratch_mutex);
         auto it = g_scratch.find(ScratchKey{device, s});
         if (it != g_scratch.end()) counters[0] = it->second.fallbacks;
+        if (device >= 0 && device < kMaxDevices && g_static_base[device])
+            counters[1] = carve(g_static_base[device], kStaticUnits).fallbacks;
     }
     for (uint32_t *c : counters) {
         if (!c) continue;
@@ -214,6 +248,19 @@ int msd_groupnorm(const void *x, void *y, const float *gamma, const float *beta,
                   void *stream) {
     return groupnorm_entry(x, nullptr, y, gamma, beta, batch, channels, hw, groups, eps, fuse_silu,
                            dtype, nullptr, stream);
+}
+
+int msd_groupnorm_noalloc(const void *x, void *y, const float *gamma, const float *beta, size_t batch,
+                          size_t channels, size_t hw, size_t groups, float eps, int fuse_silu, int dtype,
+                          void *stream) {
+    // the size check comes first so that it does not depend on a device being present
+    if (batch > kStaticUnits || groups > kStaticUnits || batch * groups > kStaticUnits)
+        return MSD_ERR_SCRATCH_LIMIT;
+    GnScratch fixed;
+    const hipError_t err = get_static_scratch(&fixed);  // a table lookup after the first call on a device
+    if (err != hipSuccess) return (int)err;
+    return groupnorm_entry(x, nullptr, y, gamma, beta, batch, channels, hw, groups, eps, fuse_silu,
+                           dtype, &fixed, stream);
 }
 
 int msd_chunk_add_groupnorm(const void *x, const void *chunk, void *y, const float *gamma,

@@ -626,7 +626,7 @@ int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma
     const size_t units = batch * groups;
     if (units == 0 || unit_size == 0) return MSD_OK;
     if (units > 0x7FFFFFFFull || unit_size > 0x7FFFFFFFull) return MSD_ERR_INVALID_VALUE;
-    if (fixed != nullptr && units > fixed->units) return MSD_ERR_INVALID_VALUE;
+    if (fixed != nullptr && units > fixed->units) return MSD_ERR_SCRATCH_LIMIT;
     if (!(aligned16(x) && aligned16(y) && hw % EPV == 0))
         return gn_generic<T>(silu, x, chunk, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
 

@@ -28,6 +28,8 @@ struct GnScratch {
 
 // Per-(device, stream) scratch, created on first use (hipMalloc + hipMemset).
 hipError_t get_scratch(hipStream_t stream, GnScratch *out);
+// The fixed scratch inside the code object (no allocation), shared by all streams of a device.
+hipError_t get_static_scratch(GnScratch *out);
 
 // Tuning overrides set through msd_set_tuning (0 = choose automatically).  Atomics: a launch
 // on one thread may read them while another thread sets them; each launch reads a knob once.

@@ -83,6 +83,11 @@ def test_argument_validation_needs_no_gpu(msd):
     assert lib.msd_geglu(p(base), p(base), rows, inner, 1, None) == 1            # in place
     assert lib.msd_geglu(p(base), p(base + 1008), rows, inner, 1, None) == 1     # out starts inside proj
     assert lib.msd_geglu(p(base + 496), p(base), rows, inner, 1, None) == 1      # proj starts inside out
+    # the entry point with the fixed scratch refuses more units than that scratch holds,
+    # before it touches a device
+    assert lib.msd_groupnorm_noalloc(p(base), p(base), p(base), p(base), 33, 64, 16, 32, 1e-5, 0, 0, None) == -2
+    assert lib.msd_groupnorm_noalloc(p(base), p(base), p(base), p(base), 2, 2050, 16, 2050, 1e-5, 0, 0, None) == -2
+    assert b"1024" in lib.msd_error_string(-2)
     assert lib.msd_gn_fallbacks(None, None, 0) == 1
     # the neighbours of the path
     assert lib.msd_linear_rows(None, None, None, None, 9, 4, 8, 0, 0, 0, None) == 1   # more than 8 rows
