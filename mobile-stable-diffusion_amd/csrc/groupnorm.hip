@@ -22,6 +22,8 @@
 // sibling's part of the input, which no workgroup overwrites before it has
 // seen every word of its unit.  The output is the same either way; a counter
 // in the scratch records how often it happened.
+#include <type_traits>
+
 #include "msd_device.h"
 #include "msd_internal.h"
 
@@ -165,75 +167,101 @@ __device__ __forceinline__ void gn_exchange(const GnScratch &scratch, const GnPa
     __syncthreads();
 }
 
+// Sum and sum of squares of a packed vector, accumulated in float32.  Half storage uses
+// v_dot2_f32_f16 (both products of a register pair are exact in float32 and are added to a
+// float32 accumulator; subnormal halves count), so the statistics never need an unpacked copy
+// of the slice.  Two accumulator pairs (even / odd registers) halve the dependent chains.
+template <typename T>
+struct Moments;
+template <>
+struct Moments<float> {
+    static __device__ __forceinline__ void add(const u32x4 &v, float (&s)[2], float (&q)[2]) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float f = __uint_as_float(v[i]);
+            s[i & 1] += f;
+            q[i & 1] = fmaf(f, f, q[i & 1]);
+        }
+    }
+};
+template <>
+struct Moments<__half> {
+    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ void add(const u32x4 &v, float (&s)[2], float (&q)[2]) {
+        const half2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t w = v[i];
+            const half2_t h = *reinterpret_cast<const half2_t *>(&w);
+            s[i & 1] = __builtin_amdgcn_fdot2(h, ones, s[i & 1], false);
+            q[i & 1] = __builtin_amdgcn_fdot2(h, h, q[i & 1], false);
+        }
+    }
+};
+
+// |mean| <= 2 sigma: the slice's M2 may be taken from the raw moments (relative error
+// below 1e-6); otherwise it is recomputed about the mean (a second pass over the registers)
+constexpr float kGnFastMoments = 4.0f;
+// |mean| <= 4 sigma of the whole unit: the epilogue may fold the mean into the offset
+constexpr float kGnFoldMean = 16.0f;
+
 // Mean and M2 = sum (x - mean)^2 of the workgroup's slice, held as K packed vectors per lane
-// (vector k of lane t is element k * blockDim.x + t of the slice; the first n_valid count).
-// Each wavefront reduces its own part in two passes with DPP only, the parts meet once in LDS
-// (one barrier), and every wavefront merges them with Chan's formula, lane l taking
-// wavefront l's entry.  FULL: every lane owns exactly K valid vectors.
+// (vector k of lane t is element k * blockDim.x + t of the slice; the first n_valid count, the
+// registers of the others hold zeros).  One pass gives sum and sum of squares (wavefront
+// reduction by DPP, the wavefronts' partial sums meet once in LDS, every wavefront adds them
+// in the same order).  M2 = sum x^2 - n mean^2 is kept when it is well conditioned; when the
+// mean is large against the spread (or the slice is constant) a second pass over the registers
+// sums (x - mean)^2 instead, so the result is as accurate as a two-pass variance either way.
+// The choice is the same in every wavefront: they all hold bit-identical sums.
 template <typename T, int K, bool FULL>
 __device__ __forceinline__ void gn_slice_stats(u32x4 (&raw)[K], uint32_t n_valid, float *red_a,
                                                float *red_b, float *red_c, float &slice_mean,
                                                float &slice_m2) {
     constexpr int EPV = Store<T>::EPV;
-    // half storage, long slices: unpack again in every pass instead of keeping K * 8 floats
-    // live; up to 8 vectors the unpacked copy fits the register file and is kept
-    constexpr bool kRepack = sizeof(T) == 2 && K > 8;
     const uint32_t tid = threadIdx.x;
     const uint32_t nt = blockDim.x;
     const uint32_t lane = tid & (kWave - 1);
-    float s = 0.0f, cnt = 0.0f;
+    const uint32_t nw = nt / kWave;
+    float s[2] = {0.0f, 0.0f}, q[2] = {0.0f, 0.0f};
 #pragma unroll
-    for (int k = 0; k < K; k++) {
-        float f[EPV];
-        Store<T>::unpack(raw[k], f);
-        float sk = 0.0f;
-#pragma unroll
-        for (int e = 0; e < EPV; e++) sk += f[e];
-        if (!FULL) {
-            const bool have = k * nt + tid < n_valid;
-            sk = have ? sk : 0.0f;
-            cnt += have ? (float)EPV : 0.0f;
-        }
-        s += sk;
-    }
-    const float wave_cnt = FULL ? (float)(kWave * K * EPV) : wave_sum(cnt);
-    const float wave_mean = wave_sum(s) / fmaxf(wave_cnt, 1.0f);
-    if (kRepack) {
-#pragma unroll
-        for (int k = 0; k < K; k++) forget(raw[k]);
-    }
-    float q = 0.0f;
-#pragma unroll
-    for (int k = 0; k < K; k++) {
-        float f[EPV];
-        Store<T>::unpack(raw[k], f);
-        float qk = 0.0f;
-#pragma unroll
-        for (int e = 0; e < EPV; e++) {
-            const float d = f[e] - wave_mean;
-            qk = fmaf(d, d, qk);
-        }
-        if (!FULL) qk = (k * nt + tid < n_valid) ? qk : 0.0f;
-        q += qk;
-    }
-    const float wave_m2 = wave_sum(q);
-    if (kRepack) {
-#pragma unroll
-        for (int k = 0; k < K; k++) forget(raw[k]);
-    }
+    for (int k = 0; k < K; k++) Moments<T>::add(raw[k], s, q);
+    const float wave_s = wave_sum(s[0] + s[1]);
+    const float wave_q = wave_sum(q[0] + q[1]);
     if (lane == 0) {
-        red_a[tid / kWave] = wave_mean;
-        red_b[tid / kWave] = wave_m2;
-        red_c[tid / kWave] = wave_cnt;
+        red_a[tid / kWave] = wave_s;
+        red_b[tid / kWave] = wave_q;
     }
     __syncthreads();
-    const bool entry = lane < nt / kWave;
-    const float m_l = entry ? red_a[lane] : 0.0f;
-    const float q_l = entry ? red_b[lane] : 0.0f;
-    const float n_l = entry ? red_c[lane] : 0.0f;
-    slice_mean = wave_sum(m_l * n_l) / (float)(n_valid * EPV);
-    const float dm = m_l - slice_mean;
-    slice_m2 = wave_sum(fmaf(n_l * dm, dm, q_l));
+    const bool entry = lane < nw;
+    const float sum_x = wave_sum(entry ? red_a[lane] : 0.0f);
+    const float sum_xx = wave_sum(entry ? red_b[lane] : 0.0f);
+    const float count = (float)(n_valid * EPV);
+    slice_mean = sum_x / count;
+    slice_m2 = sum_xx - sum_x * slice_mean;
+    // n mean^2 <= kappa M2; false also for a negative or NaN M2
+    if (!(sum_x * slice_mean <= kGnFastMoments * slice_m2)) {  // uniform over the workgroup
+        float c = 0.0f;
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            float f[EPV];
+            forget(raw[k]);  // unpack here, not once for every later use (the copies would not fit)
+            Store<T>::unpack(raw[k], f);
+            float ck = 0.0f;
+#pragma unroll
+            for (int e = 0; e < EPV; e++) {
+                const float d = f[e] - slice_mean;
+                ck = fmaf(d, d, ck);
+            }
+            if (!FULL) ck = (k * nt + tid < n_valid) ? ck : 0.0f;
+            c += ck;
+            // one vector at a time: unpacked copies of the whole slice would not fit the registers
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        const float wave_c = wave_sum(c);
+        if (lane == 0) red_c[tid / kWave] = wave_c;
+        __syncthreads();
+        slice_m2 = wave_sum(entry ? red_c[lane] : 0.0f);
+    }
 }
 
 // FULL: every lane owns exactly K vectors (no masking anywhere).
@@ -281,6 +309,14 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
             raw[k] = Store<T>::pack(f);
         }
     }
+    if (!FULL) {  // registers of lanes past the end of a ragged slice hold zeros from here on
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            const bool have = v_begin + k * nt + tid < v_end;
+#pragma unroll
+            for (int i = 0; i < 4; i++) raw[k][i] = have ? raw[k][i] : 0u;
+        }
+    }
     // per-vector channel affine: fetched up front while the data is in flight when the
     // registers allow it, otherwise just before use
     constexpr bool kPrefetchAffine = K <= 6;
@@ -322,33 +358,51 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
         rstd = stats[1];
     }
 
-    // ---- normalise from registers, per-channel affine, optional SiLU
+    // ---- normalise from registers, per-channel affine, optional SiLU.  When the unit's mean is
+    // within four standard deviations of zero it is folded into the offset,
+    // y = fma(x, a, beta - mean a) (one operation per element, error a few 1e-7 at most);
+    // otherwise y = fma(x - mean, a, beta), which stays exact for |mean| >> sigma.
+    auto epilogue = [&](auto fold_tag) {
+        constexpr bool kFold = decltype(fold_tag)::value;
 #pragma unroll
-    for (int k = 0; k < K; k++) {
-        float g_k, b_k;
-        if (kPrefetchAffine) {
-            g_k = ga[kPrefetchAffine ? k : 0];
-            b_k = be[kPrefetchAffine ? k : 0];
-        } else {
-            const uint32_t c = ch0 + fast_div(vidx[k], p.hw_vec);
-            g_k = gamma[c];
-            b_k = beta[c];
-        }
-        const float a = rstd * g_k;
-        float f[EPV];
-        Store<T>::unpack(raw[k], f);
+        for (int k = 0; k < K; k++) {
+            float g_k, b_k;
+            if (kPrefetchAffine) {
+                g_k = ga[kPrefetchAffine ? k : 0];
+                b_k = be[kPrefetchAffine ? k : 0];
+            } else {
+                const uint32_t c = ch0 + fast_div(vidx[k], p.hw_vec);
+                g_k = gamma[c];
+                b_k = beta[c];
+            }
+            const float a = rstd * g_k;
+            const float b_fold = fmaf(-mean, a, b_k);
+            float f[EPV];
+            forget(raw[k]);  // unpack here, one vector at a time
+            Store<T>::unpack(raw[k], f);
 #pragma unroll
-        for (int e = 0; e < EPV; e++) {
-            const float t = fmaf(f[e] - mean, a, b_k);
-            f[e] = SILU ? silu_f(t) : t;
+            for (int e = 0; e < EPV; e++) {
+                const float t = kFold ? fmaf(f[e], a, b_fold) : fmaf(f[e] - mean, a, b_k);
+                f[e] = SILU ? silu_f(t) : t;
+            }
+            const u32x4 packed = Store<T>::pack(f);
+            if (FULL || v_begin + k * nt + tid < v_end) store_stream(yout + vidx[k], packed);
+            // the scheduler must not start unpacking the next vectors before this one is stored:
+            // eight elements are enough independent work, and the slice stays packed until used
+            __builtin_amdgcn_sched_barrier(0);
         }
-        const u32x4 packed = Store<T>::pack(f);
-        if (FULL || v_begin + k * nt + tid < v_end) store_stream(yout + vidx[k], packed);
-    }
+    };
+    if (mean * mean * (rstd * rstd) <= kGnFoldMean)  // uniform over the workgroup
+        epilogue(std::true_type{});
+    else
+        epilogue(std::false_type{});
 }
 
+// Up to five vectors per lane (four for float storage) the kernel fits 64 registers: eight
+// wavefronts per SIMD, so two 1024-lane workgroups share a CU and one loads while the other
+// computes (what large batches need).
 template <typename T, int K, bool SILU>
-__global__ __launch_bounds__(kGnMaxThreads) void gn_slice_kernel(
+__global__ __launch_bounds__(kGnMaxThreads, (K <= (sizeof(T) == 2 ? 5 : 4) ? 8 : 4)) void gn_slice_kernel(
     const T *x, const T *chunk, T *y, const float *__restrict__ gamma,
     const float *__restrict__ beta, GnScratch scratch, GnParams p) {
     __shared__ float red_a[kGnMaxThreads / kWave];
@@ -461,6 +515,9 @@ __global__ __launch_bounds__(kGnMaxThreads) void gn_tokens_kernel(
         cl[k] = fast_div(vl, q.pos_vecs);
         pv[k] = vl - cl[k] * pvs;
         raw[k] = load_stream(xin + (size_t)cl[k] * p.hw_vec.d + slice * pvs + pv[k]);
+        const bool have = k * nt + tid < nvec;  // lanes past the end hold zeros (the statistics rely on it)
+#pragma unroll
+        for (int i = 0; i < 4; i++) raw[k][i] = have ? raw[k][i] : 0u;
     }
     const uint32_t ch0 = (unit % p.groups) * p.ch_per_group;
 

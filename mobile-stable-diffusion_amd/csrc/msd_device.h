@@ -203,28 +203,26 @@ __device__ __forceinline__ float quick_gelu_f(float x) {
     return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
-// gelu(x) = x * Phi(x), Phi(x) = 0.5 * (1 + erf(x / sqrt 2)).
-// With t = |x| and E(t) = erfc(t / sqrt 2) = 2^(t * P(t)): Phi = 0.5 E for x < 0
-// and 1 - 0.5 E otherwise, so neither tail cancels.  P is a degree-9 weighted
-// minimax fit of log2(erfc(t / sqrt 2)) / t on (0, 5.5] (relative error of E
-// below 1.4e-7; made by fit_gelu_poly.py next to this file); its leading
-// coefficient is negative, so E -> 0 beyond the fitted range without a clamp.
-// Against float64 the result is within 3.9e-7 absolute for |x| <= 32, the same
-// as the float32 expression x * 0.5 * (1 + erff(x * sqrt 0.5)).
+// gelu(x) = x * Phi(x) = max(x, 0) - h(|x|) with h(t) = 0.5 * t * erfc(t / sqrt 2), written
+// as 0.5 * (x + |x|) - t * 2^(t * P(t) - 1): neither tail cancels, one v_exp_f32, no branch.
+// P is the degree-7 fit of log2(erfc(t / sqrt 2)) / t that minimises the absolute error of h
+// (fit_gelu_poly.py next to this file prints these constants); its leading coefficient is
+// negative, so the power of two vanishes beyond the fitted range by itself.  t is clamped to
+// 64 (h is zero to float32 from 14 on) so that an infinite input gives gelu(inf) = inf and not
+// inf * 0; NaN comes through the x + |x| term.  Against float64 the result is within 2.5e-7
+// absolute everywhere (the float32 expression x * 0.5 * (1 + erff(x * sqrt 0.5)): 4.5e-7).
 __device__ __forceinline__ float gelu_erf_f(float x) {
-    const float t = fabsf(x);
-    float p = -1.824206031e-08f;
-    p = fmaf(p, t, 5.753830692e-07f);
-    p = fmaf(p, t, -7.787496543e-06f);
-    p = fmaf(p, t, 5.702746057e-05f);
-    p = fmaf(p, t, -2.093151852e-04f);
-    p = fmaf(p, t, -1.539104851e-04f);
-    p = fmaf(p, t, 7.145896088e-03f);
-    p = fmaf(p, t, -5.258353800e-02f);
-    p = fmaf(p, t, -4.591720700e-01f);
-    p = fmaf(p, t, -1.151109815e+00f);
-    const float half_e = 0.5f * __builtin_amdgcn_exp2f(p * t);
-    return x * (x < 0.0f ? half_e : 1.0f - half_e);
+    const float t = fminf(fabsf(x), 64.0f);
+    float p = -1.902064014e-06f;
+    p = fmaf(p, t, 2.805691838e-05f);
+    p = fmaf(p, t, -1.314731053e-04f);
+    p = fmaf(p, t, -2.720760531e-04f);
+    p = fmaf(p, t, 7.245421875e-03f);
+    p = fmaf(p, t, -5.262761191e-02f);
+    p = fmaf(p, t, -4.591621459e-01f);
+    p = fmaf(p, t, -1.151111007e+00f);
+    const float half_erfc = __builtin_amdgcn_exp2f(fmaf(p, t, -1.0f));
+    return fmaf(x + fabsf(x), 0.5f, -(t * half_erfc));
 }
 
 struct OpCopy {

@@ -355,7 +355,7 @@ def test_geglu_forced_vectors_per_lane(msd, orc, cuda, unroll):
 @pytest.mark.parametrize("half", [False, True], ids=["f32", "f16"])
 def test_activations(msd, orc, golden, cuda, name, half):
     fn, ref_fn = getattr(msd, name), getattr(orc, name)
-    cases = [orc.normal((2, 77, 3072), seed=4003),               # config 4 MLP hidden
+    cases = [orc.add_outliers(orc.normal((2, 77, 3072), seed=4003), seed=4003),  # config 4 MLP hidden, 1 % at +-20
              orc.add_outliers(orc.normal((77, 4096), seed=4005), seed=4005),  # the reference's size
              orc.normal((2, 1280), seed=5002),                   # SiLU on the time embedding
              golden["act_x"], orc.normal((1031,), seed=9, sigma=4.0), orc.normal((3,), seed=10)]
@@ -372,6 +372,27 @@ def test_activations(msd, orc, golden, cuda, name, half):
         assert_close_f32(got, golden["act_" + name], what=name + " fixture")
 
 
+def test_activations_on_every_finite_fp16_value(msd, orc, cuda):
+    """All 63488 finite binary16 values through SiLU, GELU, quick_GELU and as the GEGLU gate,
+    fp16 storage, against the oracle on the same values."""
+    bits = np.arange(0x10000, dtype=np.uint32).astype(np.uint16)
+    vals = bits.view(np.float16)
+    x = vals[np.isfinite(vals)].astype(np.float32)
+    assert x.size == 63488
+    xd = _to_dev(x, cuda, True)
+    for name in ("silu", "gelu", "quick_gelu"):
+        got = getattr(msd, name)(xd).float().cpu().numpy()
+        assert_close_f16(got, getattr(orc, name)(x), name + " every fp16 value")
+    for value in (1.0, -0.75, 0.001):  # value half (first), gate half (second) = every fp16 value
+        proj = np.concatenate([np.full_like(x, value), x])[None, :]
+        got = msd.geglu(_to_dev(proj, cuda, True)).float().cpu().numpy()
+        assert_close_f16(got, orc.geglu(orc.round_to_half(proj)), "geglu gate every fp16 value")
+    # fp32 storage on the same points: the plain 1e-5 criterion
+    xf = _to_dev(x, cuda)
+    for name in ("silu", "gelu", "quick_gelu"):
+        assert_close_f32(getattr(msd, name)(xf).cpu().numpy(), getattr(orc, name)(x), what=name + " fp16 grid, f32")
+
+
 def test_activation_special_values(msd, cuda):
     torch = _torch()
     x = torch.tensor([0.0, -0.0, 100.0, -100.0, 1e-30, -1e-30, 88.0, -88.0, 30.0, -30.0], device=cuda)
@@ -380,6 +401,9 @@ def test_activation_special_values(msd, cuda):
     ge = msd.gelu(x).cpu().numpy()
     assert ge[0] == 0 and ge[2] == 100.0 and abs(ge[3]) < 1e-30 and ge[6] == 88.0 and abs(ge[9]) < 1e-30
     assert np.isfinite(s).all() and np.isfinite(ge).all()
+    # non-finite inputs behave like the reference's expression x * 0.5 * (1 + erf(x / sqrt 2))
+    nf = msd.gelu(torch.tensor([float("inf"), float("nan")], device=cuda)).cpu().numpy()
+    assert nf[0] == np.inf and np.isnan(nf[1])
 
 
 # ----------------------------------------------------------------- timestep embedding + DDIM list
