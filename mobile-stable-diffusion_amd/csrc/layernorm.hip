@@ -59,10 +59,41 @@ struct Chunk {
     }
 };
 
+// Sum and sum of squares of the packed words of a chunk, accumulated in float32 (half storage:
+// v_dot2_f32_f16, whose two products are exact in float32; subnormal halves count).
+template <typename T, int NW>
+__device__ __forceinline__ void chunk_moments(const typename Words<NW>::type &v, float (&s)[2], float (&q)[2]) {
+    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+    for (int i = 0; i < NW; i++) {
+        if (sizeof(T) == 4) {
+            const float f = __uint_as_float(v[i]);
+            s[i & 1] += f;
+            q[i & 1] = fmaf(f, f, q[i & 1]);
+        } else {
+            const half2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
+            const uint32_t w = v[i];
+            const half2_t h = *reinterpret_cast<const half2_t *>(&w);
+            s[i & 1] = __builtin_amdgcn_fdot2(h, ones, s[i & 1], false);
+            q[i & 1] = __builtin_amdgcn_fdot2(h, h, q[i & 1], false);
+        }
+    }
+}
+
+// |mean| <= 2 sigma: a row's M2 may be taken from its raw moments (relative error below 1e-6)
+constexpr float kLnFastMoments = 4.0f;
+
 // A row of VPL*TL chunks (NW dwords each) is owned by TL adjacent lanes; a wavefront
-// covers 64/TL consecutive rows.  Lane (team, j) holds chunks j, j+TL, ... of its row and
-// the gamma / beta of the same columns, all requested before the first use.
-template <typename T, int NW, int VPL, int TL>
+// covers 64/TL consecutive rows.  Lane (team, j) holds chunks j, j+TL, ... of its row, all
+// requested before the first use.  One pass over the packed registers gives the row's sum and
+// sum of squares (team reduction by DPP); M2 = sum x^2 - n mean^2 is kept when it is well
+// conditioned, otherwise (a wavefront-uniform branch taken when any of its rows needs it) a
+// second pass sums (x - mean)^2.  The epilogue unpacks one chunk at a time, so the row never
+// sits in registers twice.  gamma / beta of the lane's columns are requested together with
+// the row when EARLY (short launches: one memory latency instead of two on the critical path,
+// at the price of 2 * VPL * N registers), otherwise right before use (long launches: they are
+// shared by every row and stay in the nearest cache, and more wavefronts fit a SIMD).
+template <typename T, int NW, int VPL, int TL, bool EARLY>
 __global__ __launch_bounds__(kLnMaxThreads) void ln_team_kernel(
     const T *x, const T *res, T *sum, T *y, const float *__restrict__ gamma,
     const float *__restrict__ beta, uint32_t rows, float eps, float inv_dim) {
@@ -83,15 +114,27 @@ __global__ __launch_bounds__(kLnMaxThreads) void ln_team_kernel(
     vec_t raw[VPL];
 #pragma unroll
     for (int k = 0; k < VPL; k++) raw[k] = __builtin_nontemporal_load(xin + k * TL + j);
-    vec_t raw_res[VPL];
     if (res != nullptr) {  // uniform: residual to add before the norm (the reference's elemwise_add)
         const vec_t *rin = reinterpret_cast<const vec_t *>(res) + row_chunk;
+        vec_t *sout = reinterpret_cast<vec_t *>(sum) + row_chunk;
+        vec_t raw_res[VPL];
 #pragma unroll
         for (int k = 0; k < VPL; k++) raw_res[k] = __builtin_nontemporal_load(rin + k * TL + j);
-    }
-    float g[VPL][N], b[VPL][N];
+        // x + res, rounded to the storage type and written out exactly as a separate add kernel
+        // would have left it; the norm then works on those stored values
 #pragma unroll
-    for (int k = 0; k < VPL; k++) {
+        for (int k = 0; k < VPL; k++) {
+            float f[N], r[N];
+            C::unpack(raw[k], f);
+            C::unpack(raw_res[k], r);
+#pragma unroll
+            for (int e = 0; e < N; e++) f[e] += r[e];
+            raw[k] = C::pack(f);
+            if (live) __builtin_nontemporal_store(raw[k], sout + k * TL + j);
+        }
+    }
+    // gamma / beta of chunk k's columns
+    auto affine = [&](int k, float (&g)[N], float (&b)[N]) {
         const uint32_t col = (k * TL + j) * N;
 #pragma unroll
         for (int e = 0; e < N; e += (N >= 4 ? 4 : 2)) {
@@ -100,58 +143,65 @@ __global__ __launch_bounds__(kLnMaxThreads) void ln_team_kernel(
                 const f32x4 bv = *reinterpret_cast<const f32x4 *>(beta + col + e);
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    g[k][e + i] = gv[i];
-                    b[k][e + i] = bv[i];
+                    g[e + i] = gv[i];
+                    b[e + i] = bv[i];
                 }
             } else {
                 const float2 gv = *reinterpret_cast<const float2 *>(gamma + col + e);
                 const float2 bv = *reinterpret_cast<const float2 *>(beta + col + e);
-                g[k][e] = gv.x;
-                g[k][e + 1] = gv.y;
-                b[k][e] = bv.x;
-                b[k][e + 1] = bv.y;
+                g[e] = gv.x;
+                g[e + 1] = gv.y;
+                b[e] = bv.x;
+                b[e + 1] = bv.y;
             }
         }
+    };
+    float g_all[EARLY ? VPL : 1][N], b_all[EARLY ? VPL : 1][N];
+    if (EARLY) {
+#pragma unroll
+        for (int k = 0; k < VPL; k++) affine(k, g_all[EARLY ? k : 0], b_all[EARLY ? k : 0]);
     }
-    float f[VPL][N];
-    if (res != nullptr) {
-        // x + res, rounded to the storage type and written out exactly as a separate add kernel
-        // would have left it; the norm then works on those stored values
-        vec_t *sout = reinterpret_cast<vec_t *>(sum) + row_chunk;
+    float s[2] = {0.0f, 0.0f}, q[2] = {0.0f, 0.0f};
+#pragma unroll
+    for (int k = 0; k < VPL; k++) chunk_moments<T, NW>(raw[k], s, q);
+    const float sum_x = team_sum<TL>(s[0] + s[1]);
+    const float sum_xx = team_sum<TL>(q[0] + q[1]);
+    const float mean = sum_x * inv_dim;
+    float m2 = sum_xx - sum_x * mean;
+    const bool fast = sum_x * mean <= kLnFastMoments * m2;  // false also for a negative or NaN M2
+    if (__builtin_amdgcn_ballot_w64(!fast) != 0) {  // some row of this wavefront needs the exact M2
+        float c = 0.0f;
 #pragma unroll
         for (int k = 0; k < VPL; k++) {
-            float r[N];
-            C::unpack(raw[k], f[k]);
-            C::unpack(raw_res[k], r);
+            float f[N];
+            C::unpack(raw[k], f);
 #pragma unroll
-            for (int e = 0; e < N; e++) f[k][e] += r[e];
-            raw[k] = C::pack(f[k]);
-            if (live) __builtin_nontemporal_store(raw[k], sout + k * TL + j);
+            for (int e = 0; e < N; e++) {
+                const float d = f[e] - mean;
+                c = fmaf(d, d, c);
+            }
         }
+        const float exact = team_sum<TL>(c);
+        m2 = fast ? m2 : exact;
     }
-    float s = 0.0f;
-#pragma unroll
-    for (int k = 0; k < VPL; k++) {
-        C::unpack(raw[k], f[k]);
-#pragma unroll
-        for (int e = 0; e < N; e++) s += f[k][e];
-    }
-    const float mean = team_sum<TL>(s) * inv_dim;
-    float q = 0.0f;
-#pragma unroll
-    for (int k = 0; k < VPL; k++)
-#pragma unroll
-        for (int e = 0; e < N; e++) {
-            f[k][e] -= mean;
-            q = fmaf(f[k][e], f[k][e], q);
-        }
-    const float rstd = __builtin_amdgcn_rsqf(team_sum<TL>(q) * inv_dim + eps);
+    const float rstd = __builtin_amdgcn_rsqf(m2 * inv_dim + eps);
     if (!live) return;
 #pragma unroll
     for (int k = 0; k < VPL; k++) {
-        float o[N];
+        float g[N], b[N];
+        if (EARLY) {
 #pragma unroll
-        for (int e = 0; e < N; e++) o[e] = fmaf(f[k][e] * rstd, g[k][e], b[k][e]);
+            for (int e = 0; e < N; e++) {
+                g[e] = g_all[EARLY ? k : 0][e];
+                b[e] = b_all[EARLY ? k : 0][e];
+            }
+        } else {
+            affine(k, g, b);
+        }
+        float f[N], o[N];
+        C::unpack(raw[k], f);
+#pragma unroll
+        for (int e = 0; e < N; e++) o[e] = fmaf((f[e] - mean) * rstd, g[e], b[e]);
         __builtin_nontemporal_store(C::pack(o), yout + k * TL + j);
     }
 }
@@ -200,8 +250,16 @@ void ln_launch(const T *x, const T *res, T *sum, T *y, const float *gamma, const
                                                  : (wavefronts >= 1024 ? 256u : (uint32_t)kLnThreads);
     const uint32_t rows_per_block = (kWave / TL) * (threads / kWave);
     const uint32_t blocks = (rows + rows_per_block - 1) / rows_per_block;
-    hipLaunchKernelGGL((ln_team_kernel<T, NW, VPL, TL>), dim3(blocks), dim3(threads), 0, stream, x,
-                       res, sum, y, gamma, beta, rows, eps, inv_dim);
+    // a launch of up to two wavefronts per SIMD of the chip is bound by its own latency chain:
+    // gamma / beta come with the row; beyond that by throughput: fewer registers per wavefront
+    // (measured: 8192 x 1280 fp16, 4096 wavefronts: 8.5 us late against 10.6 us early;
+    // 8192 x 320, 1024 wavefronts: 3.6 us early against 3.9 us late)
+    if (wavefronts <= 2048)
+        hipLaunchKernelGGL((ln_team_kernel<T, NW, VPL, TL, true>), dim3(blocks), dim3(threads), 0, stream, x,
+                           res, sum, y, gamma, beta, rows, eps, inv_dim);
+    else
+        hipLaunchKernelGGL((ln_team_kernel<T, NW, VPL, TL, false>), dim3(blocks), dim3(threads), 0, stream, x,
+                           res, sum, y, gamma, beta, rows, eps, inv_dim);
 }
 
 template <typename T, int NW, int TL>
