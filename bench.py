@@ -254,8 +254,15 @@ def _rotating_launch_us(torch, msd, stream, launch, xs, ys, warm=20, budget=2000
     replay = capture(torch, msd, stream, body)
     reps = max(2, int(budget // copies))
     with torch.cuda.stream(stream):
-        for _ in range(warm // copies + 1):  # at least `warm` warm-up launches
-            replay()
+        # at least `warm` warm-up launches and 20 ms of GPU work: the clocks have dropped while
+        # the host was making this case's buffers
+        t0 = time.perf_counter()
+        done = 0
+        while done < warm or time.perf_counter() - t0 < 0.02:
+            for _ in range(warm // copies + 1):
+                replay()
+            done += (warm // copies + 1) * copies
+            torch.cuda.synchronize()
         return event_time_ms(torch, replay, reps) * 1e3 / (reps * copies)
 
 
@@ -585,8 +592,14 @@ def large_batch_table(torch, msd, dev, stream):
     def measure(fn, launches):
         replay = capture(torch, msd, stream, fn)
         with torch.cuda.stream(stream):
-            replay()
-            reps = max(3, 60 // launches)
+            # the GPU has idled while the buffers were made: replay for some tens of milliseconds
+            # first so that the clocks are back up when the timed batches start
+            t0 = time.perf_counter()
+            while time.perf_counter() - t0 < 0.05:
+                for _ in range(10):
+                    replay()
+                torch.cuda.synchronize()
+            reps = max(10, 240 // launches)
             return event_time_ms(torch, replay, reps) * 1e3 / (reps * launches)
 
     cases = [("groupnorm_silu", {"batch": B, "c": 320, "hw": 4096}, B * 320 * 4096, B * 320 * 4096),
