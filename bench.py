@@ -562,6 +562,41 @@ def neighbour_table(torch, msd, dev, stream):
             rows.append(row)
             del ws
 
+    # the 22 per-ResBlock SiLU(emb) -> Linear(1280 -> Cout) projections of one step: 22 launches
+    # against one grouped launch (4 weight sets in rotation, 52 MB each in fp16)
+    couts = [c for _, c, _ in RESBLOCKS]
+    for dt, code, elt in ((torch.float16, F16, 2), (torch.float32, F32, 4)):
+        sets = 4
+        ws = [[(torch.randn(n, 1280, device=dev) * 1280 ** -0.5).to(dt) for n in couts] for _ in range(sets)]
+        bs = [torch.zeros(n, device=dev) for n in couts]
+        ys = [torch.empty(BATCH, n, device=dev, dtype=dt) for n in couts]
+        x = torch.randn(BATCH, 1280, device=dev).to(dt)
+        cnt = len(couts)
+        tables = []
+        for wset in ws:
+            tables.append(((vp * cnt)(*[w.data_ptr() for w in wset]), (vp * cnt)(*[b.data_ptr() for b in bs]),
+                           (vp * cnt)(*[y.data_ptr() for y in ys]), (ctypes.c_size_t * cnt)(*couts)))
+
+        def separate22():
+            for wset in ws:
+                for w, b, y, n in zip(wset, bs, ys, couts):
+                    assert lib.msd_linear_rows(vp(x.data_ptr()), vp(w.data_ptr()), vp(b.data_ptr()), vp(y.data_ptr()),
+                                               BATCH, n, 1280, 1, 0, code, sp()) == 0
+
+        def grouped22():
+            for wp, bp, yp, ns in tables:
+                assert lib.msd_linear_rows_grouped(vp(x.data_ptr()), wp, bp, yp, ns, cnt, BATCH, 1280, 1, 0, code,
+                                                   sp()) == 0
+        us_sep = measure(separate22, sets, 200)
+        us_grp = measure(grouped22, sets, 200)
+        nbytes = sum(couts) * 1280 * elt
+        rows.append({"kernel": "linear_rows_grouped", "what": "22 x SiLU(emb) + embed_linear of one UNet step",
+                     "shape": {"m": BATCH, "k": 1280, "n_total": sum(couts)}, "dtype": "f16" if elt == 2 else "f32",
+                     "bytes": nbytes, "us": round(us_grp, 2), "GBps": round(nbytes / us_grp / 1e3, 1),
+                     "us_22_launches": round(us_sep, 2), "speedup": round(us_sep / us_grp, 2)})
+        del ws, tables
+        torch.cuda.empty_cache()
+
     # DDIM update of the latent, batch 2 x [4, 64, 64] float32, in place
     n = BATCH * 4 * 64 * 64
     x, e = torch.randn(n, device=dev), torch.randn(n, device=dev)
@@ -645,7 +680,13 @@ def step_with_adds(torch, msd, dev, stream):
     """One UNet step of the path including the additions the reference runs right before its
     norms (the embedding add before each ResBlock out-norm, the residual add before LayerNorm 2
     and 3 of each transformer block): as separate launches in the reference's order, and
-    folded into the norm kernels.  Same buffers, graph-replayed."""
+    folded into the norm kernels.  Same buffers, graph-replayed.
+
+    A second pair adds the Linear layers on the embedding rows that the reference runs between
+    those launches (time_embed_0 / SiLU / time_embed_2, M/UNetModel.cpp:1107-1120, and SiLU(emb)
+    -> embed_linear in every ResBlock, M/nn/ResBlock.cpp:173-183, whose output is what the
+    embedding add adds): every launch separate, against SiLU folded into the Linear kernels and
+    the 22 projections as ONE grouped launch ahead of the blocks."""
     import ctypes
     vp = ctypes.c_void_p
     lib = msd.load_library()
@@ -666,18 +707,52 @@ def step_with_adds(torch, msd, dev, stream):
         return affine[c]
 
     separate, fused = [], []  # lists of (fn, args)
-    out_norm, ln_count = False, 0
+    separate_emb, fused_emb = [], []  # the same with the embedding-row Linear layers
+    # embedding path: sinusoid [2, 320] -> h [2, 1280] -> emb [2, 1280] -> per ResBlock [2, Cout]
+    couts = [c for _, c, _ in RESBLOCKS]
+    temb_out = torch.empty((BATCH, 320), device=dev, dtype=torch.float16)
+    h_buf = torch.empty((BATCH, 1280), device=dev, dtype=torch.float16)
+    emb_buf = torch.empty((BATCH, 1280), device=dev, dtype=torch.float16)
+    emb_act = torch.empty((BATCH, 1280), device=dev, dtype=torch.float16)
+    w_te0, w_te2 = randn(1280, 320) * 320 ** -0.5, randn(1280, 1280) * 1280 ** -0.5
+    w_res = [randn(c, 1280) * 1280 ** -0.5 for c in couts]
+    b_te = 0.1 * randn(1280, dtype=torch.float32)
+    b_res = [0.1 * randn(c, dtype=torch.float32) for c in couts]
+    proj = [torch.empty((BATCH, c), device=dev, dtype=torch.float16) for c in couts]
+    keep += [temb_out, h_buf, emb_buf, emb_act, w_te0, w_te2, b_te] + w_res + b_res + proj
+    cnt = len(couts)
+    group_tables = ((vp * cnt)(*[w.data_ptr() for w in w_res]), (vp * cnt)(*[b.data_ptr() for b in b_res]),
+                    (vp * cnt)(*[y.data_ptr() for y in proj]), (ctypes.c_size_t * cnt)(*couts))
+    keep.append(group_tables)
+
+    def lin(x, w, b, y, n, k, act_in, act_out):
+        return (lib.msd_linear_rows, (vp(x.data_ptr()), vp(w.data_ptr()), vp(b.data_ptr()), vp(y.data_ptr()), BATCH, n, k,
+                                      act_in, act_out, F16))
+    out_norm, ln_count, res_index = False, 0, -1
     for kind, p in step_layers():
         if kind == "temb":
             t = torch.randint(0, 1000, (BATCH,), device=dev, dtype=torch.int64, generator=g)
-            out = torch.empty((BATCH, p["dim"]), device=dev, dtype=torch.float16)
-            keep += [t, out]
-            call = (lib.msd_timestep_embedding, (vp(t.data_ptr()), vp(out.data_ptr()), BATCH, p["dim"], 10000.0, F16))
-            separate.append(call), fused.append(call)
+            keep += [t]
+            call = (lib.msd_timestep_embedding, (vp(t.data_ptr()), vp(temb_out.data_ptr()), BATCH, p["dim"], 10000.0, F16))
+            for lst in (separate, fused, separate_emb, fused_emb):
+                lst.append(call)
         elif kind == "silu":
             x = randn(p["n"])
             call = (lib.msd_silu, (vp(x.data_ptr()), vp(x.data_ptr()), p["n"], F16))
             separate.append(call), fused.append(call)
+            if res_index < 0:  # the time-embedding MLP: Linear, SiLU, Linear
+                separate_emb.append(lin(temb_out, w_te0, b_te, h_buf, 1280, 320, 0, 0))
+                separate_emb.append((lib.msd_silu, (vp(h_buf.data_ptr()), vp(h_buf.data_ptr()), BATCH * 1280, F16)))
+                separate_emb.append(lin(h_buf, w_te2, b_te, emb_buf, 1280, 1280, 0, 0))
+                fused_emb.append(lin(temb_out, w_te0, b_te, h_buf, 1280, 320, 0, 1))
+                fused_emb.append(lin(h_buf, w_te2, b_te, emb_buf, 1280, 1280, 0, 0))
+                fused_emb.append((lib.msd_linear_rows_grouped, (vp(emb_buf.data_ptr()),) + group_tables +
+                                  (cnt, BATCH, 1280, 1, 0, F16)))
+            else:              # a ResBlock's SiLU(emb) -> embed_linear (already done by the grouped launch)
+                separate_emb.append((lib.msd_silu, (vp(emb_buf.data_ptr()), vp(emb_act.data_ptr()), BATCH * 1280, F16)))
+                separate_emb.append(lin(emb_act, w_res[res_index], b_res[res_index], proj[res_index], couts[res_index],
+                                        1280, 0, 0))
+            res_index += 1
             out_norm = True  # the next GroupNorm is the ResBlock's out-norm (after the embedding add)
         elif kind == "gn_silu":
             c, hw = p["c"], p["hw"]
@@ -694,10 +769,16 @@ def step_with_adds(torch, msd, dev, stream):
                 separate.append((lib.msd_chunkwise_add, (xp, ep, xp, BATCH * c * hw, hw, F16)))
                 separate.append((lib.msd_groupnorm, (xp, yp, gp, bp, BATCH, c, hw, 32, 1e-5, 1, F16)))
                 fused.append((lib.msd_chunk_add_groupnorm, (xp, ep, yp, gp, bp, BATCH, c, hw, 32, 1e-5, 1, F16)))
+                pp = vp(proj[res_index - 1].data_ptr())  # this ResBlock's projection of the embedding
+                assert couts[res_index - 1] == c
+                separate_emb.append((lib.msd_chunkwise_add, (xp, pp, xp, BATCH * c * hw, hw, F16)))
+                separate_emb.append((lib.msd_groupnorm, (xp, yp, gp, bp, BATCH, c, hw, 32, 1e-5, 1, F16)))
+                fused_emb.append((lib.msd_chunk_add_groupnorm, (xp, pp, yp, gp, bp, BATCH, c, hw, 32, 1e-5, 1, F16)))
                 out_norm = False
             else:
                 call = (lib.msd_groupnorm, (xp, yp, gp, bp, BATCH, c, hw, 32, 1e-5, 1, F16))
-                separate.append(call), fused.append(call)
+                for lst in (separate, fused, separate_emb, fused_emb):
+                    lst.append(call)
         elif kind == "ln":
             rows, dim = p["rows"], p["dim"]
             x, y = randn(rows, dim), torch.empty((rows, dim), device=dev, dtype=torch.float16)
@@ -706,13 +787,16 @@ def step_with_adds(torch, msd, dev, stream):
             xp, yp, gp, bp = vp(x.data_ptr()), vp(y.data_ptr()), vp(ga.data_ptr()), vp(be.data_ptr())
             if ln_count % 3 == 0:  # LayerNorm 1 of a block has no add in front
                 call = (lib.msd_layernorm, (xp, yp, gp, bp, rows, dim, 1e-5, F16))
-                separate.append(call), fused.append(call)
+                for lst in (separate, fused, separate_emb, fused_emb):
+                    lst.append(call)
             else:
                 res = randn(rows, dim)
                 rp = vp(res.data_ptr())
-                separate.append((lib.msd_elemwise_add, (xp, rp, xp, rows * dim, F16)))
-                separate.append((lib.msd_layernorm, (xp, yp, gp, bp, rows, dim, 1e-5, F16)))
-                fused.append((lib.msd_add_layernorm, (xp, rp, xp, yp, gp, bp, rows, dim, 1e-5, F16)))
+                for lst in (separate, separate_emb):
+                    lst.append((lib.msd_elemwise_add, (xp, rp, xp, rows * dim, F16)))
+                    lst.append((lib.msd_layernorm, (xp, yp, gp, bp, rows, dim, 1e-5, F16)))
+                for lst in (fused, fused_emb):
+                    lst.append((lib.msd_add_layernorm, (xp, rp, xp, yp, gp, bp, rows, dim, 1e-5, F16)))
             ln_count += 1
         else:
             rows, inner = p["rows"], p["inner"]
@@ -720,7 +804,8 @@ def step_with_adds(torch, msd, dev, stream):
             y = torch.empty((rows, inner), device=dev, dtype=torch.float16)
             keep.append(y)
             call = (lib.msd_geglu, (vp(x.data_ptr()), vp(y.data_ptr()), rows, inner, F16))
-            separate.append(call), fused.append(call)
+            for lst in (separate, fused, separate_emb, fused_emb):
+                lst.append(call)
 
     def runner(calls):
         def run():
@@ -730,7 +815,8 @@ def step_with_adds(torch, msd, dev, stream):
         return run
 
     out = {}
-    for name, calls in (("separate", separate), ("fused", fused)):
+    for name, calls in (("separate", separate), ("fused", fused), ("separate_emb", separate_emb),
+                        ("fused_emb", fused_emb)):
         replay = capture(torch, msd, stream, runner(calls))
         with torch.cuda.stream(stream):
             for _ in range(5):
@@ -738,7 +824,11 @@ def step_with_adds(torch, msd, dev, stream):
             out[name] = event_time_ms(torch, replay, 50) / 50
     return {"launches_separate": len(separate), "launches_fused": len(fused),
             "ms_separate": round(out["separate"], 4), "ms_fused": round(out["fused"], 4),
-            "speedup": round(out["separate"] / out["fused"], 3)}
+            "speedup": round(out["separate"] / out["fused"], 3),
+            "with_embedding_linears": {
+                "launches_separate": len(separate_emb), "launches_fused_grouped": len(fused_emb),
+                "ms_separate": round(out["separate_emb"], 4), "ms_fused_grouped": round(out["fused_emb"], 4),
+                "speedup": round(out["separate_emb"] / out["fused_emb"], 3)}}
 
 
 def cpu_baseline(total_bytes, budget_s=24.0):

@@ -245,6 +245,19 @@ int msd_linear_rows(const void *x, const void *weight, const float *bias, void *
                     size_t n, size_t k, int act_in, int act_out, int dtype, void *stream);
 
 /*
+ * `count` such layers on the SAME rows x in one launch: ys[i][m, ns[i]] = act_out(act_in(x) .
+ * weights[i][ns[i], k]^T + biases[i]).  weights, biases, ys and ns are host arrays of `count`
+ * entries (device pointers / sizes); biases or any biases[i] may be NULL.  Replaces the 22
+ * `silu(emb)` + `embed_linear->forward` pairs of one UNet step (M/nn/ResBlock.cpp:173-183),
+ * which all read the one embedding that UNetModel::forward computes before its first block
+ * (M/UNetModel.cpp:1107-1120), by one launch ahead of the blocks; each ys[i] equals what its
+ * own msd_linear_rows call gives, bit for bit.  No ys[i] may overlap x.
+ */
+int msd_linear_rows_grouped(const void *x, const void *const *weights, const float *const *biases,
+                            void *const *ys, const size_t *ns, size_t count, size_t m, size_t k,
+                            int act_in, int act_out, int dtype, void *stream);
+
+/*
  * Row softmax over the last dimension of [rows, cols]; y may alias x (every reference
  * call site is in place).  Replaces the softmax kernel K/util.cl:150-187 enqueued by
  * CrossAttention::forward (M/nn/CrossAttention.cpp:362-377) and AttnBlock::forward

@@ -28,7 +28,7 @@ C_ABI_SYMBOLS = (
     "msd_silu", "msd_gelu", "msd_quick_gelu", "msd_timestep_embedding", "msd_ddim_timesteps",
     "msd_elemwise_add", "msd_chunkwise_add", "msd_chunk_add_groupnorm", "msd_add_layernorm", "msd_copy",
     "msd_groupnorm_tokens", "msd_permute_0_2_1",
-    "msd_linear_rows", "msd_softmax", "msd_alphas_cumprod", "msd_ddim_schedule", "msd_ddim_update",
+    "msd_linear_rows", "msd_linear_rows_grouped", "msd_softmax", "msd_alphas_cumprod", "msd_ddim_schedule", "msd_ddim_update",
 )
 ACT_NONE, ACT_SILU = 0, 1
 
@@ -77,6 +77,8 @@ def load_library(path=None):
     lib.msd_ddim_timesteps.argtypes = [it, ctypes.POINTER(ctypes.c_int), it]
     lib.msd_linear_rows.argtypes = [vp, vp, vp, vp, sz, sz, sz, it, it, it, vp]
     lib.msd_softmax.argtypes = [vp, vp, sz, sz, it, it, vp]
+    lib.msd_linear_rows_grouped.argtypes = [vp, ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(vp),
+                                            ctypes.POINTER(sz), sz, sz, sz, it, it, it, vp]
     flp, inp = ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_int)
     lib.msd_alphas_cumprod.argtypes = [flp]
     lib.msd_ddim_schedule.argtypes = [it, inp, flp, flp, flp, it]
@@ -305,6 +307,30 @@ def linear_rows(x, weight, bias=None, act_in=ACT_NONE, act_out=ACT_NONE, out=Non
     check(load_library().msd_linear_rows(_dev(x), _dev(weight), bp, _same(out, x, m * n, "out"), m, n, k, act_in, act_out,
                                          _dtype_code(x), _stream()))
     return out
+
+
+def linear_rows_grouped(x, weights, biases=None, act_in=ACT_NONE, act_out=ACT_NONE):
+    """One launch for several Linear layers on the same x [m <= 8, k]: weights[i] is [n_i, k] in
+    x's dtype, biases[i] float32 [n_i] or None -> list of [m, n_i] tensors."""
+    import torch
+    m, k = x.shape
+    count = len(weights)
+    outs, wp, bp, yp, ns = [], (ctypes.c_void_p * count)(), (ctypes.c_void_p * count)(), \
+        (ctypes.c_void_p * count)(), (ctypes.c_size_t * count)()
+    for i, w in enumerate(weights):
+        if w.dim() != 2 or w.shape[1] != k or w.dtype != x.dtype or w.device != x.device:
+            raise MsdError("weights[%d] must be [n, %d] in the dtype and on the device of x" % (i, k))
+        n = w.shape[0]
+        out = torch.empty((m, n), dtype=x.dtype, device=x.device)
+        outs.append(out)
+        wp[i], yp[i], ns[i] = w.data_ptr() if w.numel() else None, out.data_ptr() if out.numel() else None, n
+        b = biases[i] if biases is not None else None
+        bp[i] = _affine(b, n, x, "biases[%d]" % i).value if b is not None else None
+        if not w.is_contiguous():
+            raise MsdError("expected contiguous weights")
+    check(load_library().msd_linear_rows_grouped(_dev(x), wp, bp, yp, ns, count, m, k, act_in, act_out,
+                                                 _dtype_code(x), _stream()))
+    return outs
 
 
 def softmax(x, stable=False, out=None):

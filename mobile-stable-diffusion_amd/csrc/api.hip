@@ -408,6 +408,25 @@ int msd_linear_rows(const void *x, const void *weight, const float *bias, void *
     return linear_rows_dispatch<__half>(x, weight, bias, y, m, n, k, act_in, act_out, s);
 }
 
+int msd_linear_rows_grouped(const void *x, const void *const *weights, const float *const *biases,
+                            void *const *ys, const size_t *ns, size_t count, size_t m, size_t k,
+                            int act_in, int act_out, int dtype, void *stream) {
+    if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
+    if ((act_in != MSD_ACT_NONE && act_in != MSD_ACT_SILU) ||
+        (act_out != MSD_ACT_NONE && act_out != MSD_ACT_SILU))
+        return MSD_ERR_INVALID_VALUE;
+    if (m > 8) return MSD_ERR_INVALID_VALUE;
+    if (count != 0 && (!weights || !ys || !ns)) return MSD_ERR_INVALID_VALUE;
+    for (size_t i = 0; i < count && m != 0; i++) {
+        if (ns[i] == 0) continue;
+        if (!ys[i] || (k != 0 && (!x || !weights[i])) || x == ys[i]) return MSD_ERR_INVALID_VALUE;
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == MSD_DTYPE_F32)
+        return linear_rows_grouped_dispatch<float>(x, weights, biases, ys, ns, count, m, k, act_in, act_out, s);
+    return linear_rows_grouped_dispatch<__half>(x, weights, biases, ys, ns, count, m, k, act_in, act_out, s);
+}
+
 int msd_softmax(const void *x, void *y, size_t rows, size_t cols, int stable, int dtype,
                 void *stream) {
     if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;

@@ -23,14 +23,14 @@ namespace {
 // ---------------------------------------------------------------------------
 
 template <typename T, int M, int CPW>
-__global__ __launch_bounds__(kWave) void linear_rows_kernel(
-    const T *__restrict__ x, const T *__restrict__ w, const float *__restrict__ bias,
-    T *__restrict__ y, uint32_t m, uint32_t n, uint32_t kvecs, int act_in, int act_out) {
+__device__ __forceinline__ void linear_rows_body(const T *__restrict__ x, const T *__restrict__ w,
+                                                 const float *__restrict__ bias, T *__restrict__ y,
+                                                 uint32_t m, uint32_t n, uint32_t kvecs, int act_in,
+                                                 int act_out, uint32_t col0) {
     constexpr int EPV = Store<T>::EPV;
     // pieces per lane per round: one round covers k = 2048 (float with more than 4 rows: 1024)
     constexpr int kLinRound = (sizeof(T) == 4 && M <= 4) ? 8 : 4;
     const uint32_t lane = threadIdx.x;
-    const uint32_t col0 = blockIdx.x * CPW;
     const u32x4 *xin = reinterpret_cast<const u32x4 *>(x);
     const u32x4 *win = reinterpret_cast<const u32x4 *>(w);
     float acc[CPW][M];
@@ -89,6 +89,38 @@ __global__ __launch_bounds__(kWave) void linear_rows_kernel(
             Store<T>::store1(y + (size_t)lane * n + col, r);
         }
     }
+}
+
+template <typename T, int M, int CPW>
+__global__ __launch_bounds__(kWave) void linear_rows_kernel(
+    const T *__restrict__ x, const T *__restrict__ w, const float *__restrict__ bias,
+    T *__restrict__ y, uint32_t m, uint32_t n, uint32_t kvecs, int act_in, int act_out) {
+    linear_rows_body<T, M, CPW>(x, w, bias, y, m, n, kvecs, act_in, act_out, blockIdx.x * CPW);
+}
+
+// Several Linear layers on the same rows x in one launch (the per-ResBlock projections of the
+// time embedding all read the same [m, k] embedding): the problems' workgroups are laid end to
+// end, a workgroup finds its problem by walking the table of first workgroups (at most
+// kLinGroupMax entries, passed by value with the launch), then runs the same code as a single
+// launch would, so each problem's result is that of its own msd_linear_rows call bit for bit.
+constexpr int kLinGroupMax = 32;
+struct LinearGroup {
+    const void *w[kLinGroupMax];
+    const float *bias[kLinGroupMax];
+    void *y[kLinGroupMax];
+    uint32_t n[kLinGroupMax];
+    uint32_t first_block[kLinGroupMax + 1];  // first_block[count] = number of workgroups
+    uint32_t count;
+};
+
+template <typename T, int M, int CPW>
+__global__ __launch_bounds__(kWave) void linear_rows_grouped_kernel(const T *__restrict__ x, LinearGroup g,
+                                                                    uint32_t m, uint32_t kvecs, int act_in,
+                                                                    int act_out) {
+    uint32_t p = 0;
+    while (p + 1 < g.count && blockIdx.x >= g.first_block[p + 1]) p++;  // uniform: scalar loop
+    linear_rows_body<T, M, CPW>(x, static_cast<const T *>(g.w[p]), g.bias[p], static_cast<T *>(g.y[p]), m,
+                                g.n[p], kvecs, act_in, act_out, (blockIdx.x - g.first_block[p]) * CPW);
 }
 
 constexpr int kLinThreads = 256;  // workgroup of the scalar kernel below
@@ -433,6 +465,74 @@ int linear_rows_dispatch(const void *xv, const void *wv, const float *bias, void
     return launch_status();
 }
 
+namespace {
+
+template <typename T, int M>
+void linear_grouped_launch(const T *x, const LinearGroup &g, uint32_t m, uint32_t k, int act_in, int act_out,
+                           int cpw, hipStream_t stream) {
+    constexpr int EPV = Store<T>::EPV;
+    const uint32_t blocks = g.first_block[g.count];
+    if (cpw == 2)
+        hipLaunchKernelGGL((linear_rows_grouped_kernel<T, M, 2>), dim3(blocks), dim3(kWave), 0, stream, x, g, m,
+                           k / EPV, act_in, act_out);
+    else
+        hipLaunchKernelGGL((linear_rows_grouped_kernel<T, M, 1>), dim3(blocks), dim3(kWave), 0, stream, x, g, m,
+                           k / EPV, act_in, act_out);
+}
+
+}  // namespace
+
+template <typename T>
+int linear_rows_grouped_dispatch(const void *xv, const void *const *ws, const float *const *biases,
+                                 void *const *ys, const size_t *ns, size_t count, size_t m, size_t k,
+                                 int act_in, int act_out, hipStream_t stream) {
+    constexpr int EPV = Store<T>::EPV;
+    const T *x = static_cast<const T *>(xv);
+    if (m == 0 || count == 0) return MSD_OK;
+    if (m > 8 || k > 0x7FFFFFFFull) return MSD_ERR_INVALID_VALUE;
+    bool vectors = k != 0 && k % EPV == 0 && aligned16(x);
+    for (size_t i = 0; i < count; i++) {
+        if (ns[i] > 0x7FFFFFFFull) return MSD_ERR_INVALID_VALUE;
+        vectors = vectors && aligned16(ws[i]);
+    }
+    if (!vectors) {  // odd k or alignment: one launch of the scalar kernel per problem
+        for (size_t i = 0; i < count; i++) {
+            const int rc = linear_rows_dispatch<T>(xv, ws[i], biases ? biases[i] : nullptr, ys[i], m, ns[i], k,
+                                                   act_in, act_out, stream);
+            if (rc != MSD_OK) return rc;
+        }
+        return MSD_OK;
+    }
+    const uint32_t m_pad = m <= 1 ? 1 : m <= 2 ? 2 : m <= 4 ? 4 : 8;
+    const int cpw = act_in ? 2 : 1;  // as the single launch: two columns share the activated x
+    for (size_t base = 0; base < count; base += kLinGroupMax) {
+        LinearGroup g;
+        g.count = 0;
+        uint32_t blocks = 0;
+        for (size_t i = base; i < count && i < base + kLinGroupMax; i++) {
+            if (ns[i] == 0) continue;
+            const uint32_t slot = g.count++;
+            g.w[slot] = ws[i];
+            g.bias[slot] = biases ? biases[i] : nullptr;
+            g.y[slot] = ys[i];
+            g.n[slot] = (uint32_t)ns[i];
+            g.first_block[slot] = blocks;
+            blocks += (uint32_t)((ns[i] + cpw - 1) / cpw);
+        }
+        if (g.count == 0) continue;
+        g.first_block[g.count] = blocks;
+        switch (m_pad) {
+            case 1: linear_grouped_launch<T, 1>(x, g, (uint32_t)m, (uint32_t)k, act_in, act_out, cpw, stream); break;
+            case 2: linear_grouped_launch<T, 2>(x, g, (uint32_t)m, (uint32_t)k, act_in, act_out, cpw, stream); break;
+            case 4: linear_grouped_launch<T, 4>(x, g, (uint32_t)m, (uint32_t)k, act_in, act_out, cpw, stream); break;
+            default: linear_grouped_launch<T, 8>(x, g, (uint32_t)m, (uint32_t)k, act_in, act_out, cpw, stream); break;
+        }
+        const int rc = launch_status();
+        if (rc != MSD_OK) return rc;
+    }
+    return MSD_OK;
+}
+
 template <typename T>
 int softmax_dispatch(const void *xv, void *yv, size_t rows, size_t cols, int stable, hipStream_t stream) {
     constexpr int EPV = Store<T>::EPV;
@@ -503,6 +603,10 @@ int ddim_update_dispatch(const void *xv, const void *ev, void *yv, size_t n, flo
 
 template int linear_rows_dispatch<float>(const void *, const void *, const float *, void *, size_t, size_t, size_t, int, int, hipStream_t);
 template int linear_rows_dispatch<__half>(const void *, const void *, const float *, void *, size_t, size_t, size_t, int, int, hipStream_t);
+template int linear_rows_grouped_dispatch<float>(const void *, const void *const *, const float *const *, void *const *,
+                                                 const size_t *, size_t, size_t, size_t, int, int, hipStream_t);
+template int linear_rows_grouped_dispatch<__half>(const void *, const void *const *, const float *const *, void *const *,
+                                                  const size_t *, size_t, size_t, size_t, int, int, hipStream_t);
 template int softmax_dispatch<float>(const void *, void *, size_t, size_t, int, hipStream_t);
 template int softmax_dispatch<__half>(const void *, void *, size_t, size_t, int, hipStream_t);
 template int ddim_update_dispatch<float>(const void *, const void *, void *, size_t, float, float, float, hipStream_t);

@@ -80,6 +80,11 @@ int temb_dispatch(const int64_t *timesteps, void *out, size_t batch, size_t dim,
 template <typename T>
 int linear_rows_dispatch(const void *x, const void *w, const float *bias, void *y, size_t m, size_t n,
                          size_t k, int act_in, int act_out, hipStream_t stream);
+// `count` Linear layers on the same rows x; ws / biases / ys / ns are host arrays
+template <typename T>
+int linear_rows_grouped_dispatch(const void *x, const void *const *ws, const float *const *biases,
+                                 void *const *ys, const size_t *ns, size_t count, size_t m, size_t k,
+                                 int act_in, int act_out, hipStream_t stream);
 template <typename T>
 int softmax_dispatch(const void *x, void *y, size_t rows, size_t cols, int stable, hipStream_t stream);
 template <typename T>

@@ -93,6 +93,8 @@ def test_argument_validation_needs_no_gpu(msd):
     assert lib.msd_linear_rows(None, None, None, None, 9, 4, 8, 0, 0, 0, None) == 1   # more than 8 rows
     assert lib.msd_linear_rows(None, None, None, None, 2, 4, 8, 0, 0, 0, None) == 1   # null pointers
     assert lib.msd_linear_rows(None, None, None, None, 2, 4, 8, 3, 0, 0, None) == 1   # unknown activation
+    assert lib.msd_linear_rows_grouped(None, None, None, None, None, 2, 2, 8, 0, 0, 0, None) == 1  # null tables
+    assert lib.msd_linear_rows_grouped(None, None, None, None, None, 0, 2, 8, 0, 0, 0, None) == 0  # nothing to do
     assert lib.msd_softmax(None, None, 4, 77, 0, 0, None) == 1
     assert lib.msd_softmax(None, None, 0, 77, 0, 0, None) == 0                        # empty: nothing to do
     assert lib.msd_ddim_update(None, None, None, 16, 0.5, 0.5, 0.7, 0, None) == 1

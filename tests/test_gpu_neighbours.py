@@ -94,6 +94,71 @@ def test_linear_unaligned_views_and_rejections(msd, orc, cuda):
     assert lib.msd_linear_rows(xd.data_ptr(), wd.data_ptr(), None, out.data_ptr(), 0, 20, 328, 0, 0, 0, s) == 0
 
 
+# output channels of the 22 ResBlocks of one UNet step, in execution order (M/UNetModel.cpp:86-1018)
+RESBLOCK_COUT = [320, 320, 640, 640, 1280, 1280, 1280, 1280, 1280, 1280, 1280, 1280, 1280, 1280, 1280, 1280,
+                 640, 640, 640, 320, 320, 320]
+
+
+@pytest.mark.parametrize("half", [False, True], ids=["f32", "f16"])
+def test_grouped_linear_runs_the_22_resblock_projections_in_one_launch(msd, orc, cuda, half):
+    """SiLU(emb) -> Linear(1280 -> Cout) of every ResBlock (M/nn/ResBlock.cpp:173-183) as one
+    launch: each output against the oracle and bit for bit against its own msd_linear_rows call."""
+    torch = _torch()
+    emb = orc.normal((2, 1280), seed=7500, sigma=1.5)
+    ws = [orc.normal((n, 1280), seed=7501 + i, sigma=1280 ** -0.5) for i, n in enumerate(RESBLOCK_COUT)]
+    bs = [orc.normal((n,), seed=7601 + i, sigma=0.1) for i, n in enumerate(RESBLOCK_COUT)]
+    if half:
+        emb, ws = orc.round_to_half(emb), [orc.round_to_half(w) for w in ws]
+    ed = _to_dev(emb, cuda, half)
+    wd = [_to_dev(w, cuda, half) for w in ws]
+    bd = [_to_dev(b, cuda) for b in bs]
+    outs = msd.linear_rows_grouped(ed, wd, bd, act_in=msd.ACT_SILU)
+    assert len(outs) == 22
+    for i, (o, w, b) in enumerate(zip(outs, ws, bs)):
+        single = msd.linear_rows(ed, wd[i], bd[i], act_in=msd.ACT_SILU)
+        assert torch.equal(o, single), "problem %d differs from its own launch" % i
+        ref = orc.linear(orc.silu(emb), w, b)
+        if half:
+            assert_close_f16(o.float().cpu().numpy(), ref, "grouped linear f16")
+        else:
+            assert_close_f32(o.cpu().numpy(), ref, what="grouped linear %d" % i)
+
+
+def test_grouped_linear_edge_cases(msd, orc, cuda):
+    torch = _torch()
+    # more problems than one launch's table holds, empty problems, missing biases, no activation
+    ns = [3, 0, 130, 1, 64] * 8
+    x = orc.normal((3, 96), seed=7700)
+    ws = [orc.normal((n, 96), seed=7701 + i, sigma=0.1) for i, n in enumerate(ns)]
+    bs = [orc.normal((n,), seed=7801 + i) if i % 3 else None for i, n in enumerate(ns)]
+    xd = _to_dev(x, cuda)
+    outs = msd.linear_rows_grouped(xd, [_to_dev(w, cuda) for w in ws],
+                                   [_to_dev(b, cuda) if b is not None else None for b in bs], act_out=msd.ACT_SILU)
+    for o, w, b, n in zip(outs, ws, bs, ns):
+        assert o.shape == (3, n)
+        if n:
+            assert_close_f32(o.cpu().numpy(), orc.silu(orc.linear(x, w, b)), what="grouped edge")
+    # k that does not vectorise: falls back to one scalar launch per problem, same results
+    x2 = orc.normal((2, 77), seed=7900)
+    w2 = [orc.normal((5, 77), seed=7901), orc.normal((9, 77), seed=7902)]
+    o2 = msd.linear_rows_grouped(_to_dev(x2, cuda), [_to_dev(w, cuda) for w in w2])
+    for o, w in zip(o2, w2):
+        assert_close_f32(o.cpu().numpy(), orc.linear(x2, w), what="grouped odd k")
+    assert msd.linear_rows_grouped(xd, []) == []
+    # rejections: more than 8 rows, an output that is the input
+    lib = msd.load_library()
+    import ctypes
+    vp = ctypes.c_void_p
+    arr = lambda *v: (vp * len(v))(*v)
+    one = (ctypes.c_size_t * 1)(96)
+    s = torch.cuda.current_stream().cuda_stream
+    wdev = _to_dev(ws[2], cuda)
+    assert lib.msd_linear_rows_grouped(xd.data_ptr(), arr(wdev.data_ptr()), None, arr(xd.data_ptr()), one, 1, 3, 96,
+                                       0, 0, 0, s) == 1
+    assert lib.msd_linear_rows_grouped(xd.data_ptr(), arr(wdev.data_ptr()), None, arr(outs[2].data_ptr()), one, 1, 9,
+                                       96, 0, 0, 0, s) == 1
+
+
 def test_time_embedding_mlp_chain(msd, orc, cuda):
     """timestep -> sinusoid -> Linear+SiLU -> Linear -> SiLU+Linear, as one UNet step runs it."""
     torch = _torch()
