@@ -651,6 +651,8 @@ GnPlan plan_slice(uint32_t vecs, uint32_t split, uint32_t force_threads, uint32_
         if (pl.threads == 0) pl.threads = kGnMaxThreads;
     } else if (vecs > 512u * 5u || (split > 1 && vecs >= 960))  // slices of a cut unit: 2 - 3 % faster
         pl.threads = kGnMaxThreads;
+    else if (split == 1 && vecs >= 256 && vecs <= 704 && vecs % kWave == 0)
+        pl.threads = vecs;  // one vector per lane, nothing masked: 3 % faster for the 8 x 8 maps
     else if (vecs >= 256)
         pl.threads = 512;
     else
