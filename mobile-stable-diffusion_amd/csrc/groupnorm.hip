@@ -32,9 +32,13 @@ namespace msd {
 namespace {
 
 constexpr int kGnMaxThreads = 1024;
-constexpr int kGnMaxK = 16;
+constexpr int kGnMaxK = 20;        // vectors per lane; the largest only for slices it fits exactly
+constexpr int kGnMaxRaggedK = 16;  // the largest with code for a ragged slice
 constexpr uint32_t kGnSpinLimit = 2048;  // default poll limit: about half a microsecond per poll
 constexpr int kGenericThreads = 256;
+constexpr size_t kChipCus = 256;  // compute units of an MI355X
+constexpr int kGnPrefetchAffineK = 6;       // vectors per lane up to which gamma / beta are kept in registers
+constexpr uint32_t kGnLdsChannels = 1024;  // channels per group the LDS copy of gamma / beta has room for
 
 struct GnParams {
     uint32_t vec_per_unit;   // 16-byte vectors per unit
@@ -271,7 +275,7 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
                                         const float *__restrict__ beta, const GnScratch &scratch,
                                         const GnParams &p, uint32_t unit, uint32_t slice,
                                         uint32_t v_begin, uint32_t v_end, float *red_a,
-                                        float *red_b, float *red_c, float *stats) {
+                                        float *red_b, float *red_c, float *stats, float *aff) {
     constexpr int EPV = Store<T>::EPV;
     const uint32_t tid = threadIdx.x;
     const uint32_t nt = blockDim.x;
@@ -286,13 +290,29 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
     // ---- the slice goes into registers.  Lanes past the end of a ragged slice re-read its
     // last vector (a valid address) and are masked later: no load sits behind a branch.
     u32x4 raw[K];
-    uint32_t vidx[K];
+    // Index of a lane's k-th vector inside the unit, and its address.  Both are recomputed
+    // from the lane number wherever they are needed (a few instructions) instead of being kept
+    // in registers per vector; `lane_again()` returns the lane number as a value the compiler
+    // cannot tie to earlier computations, so it cannot decide otherwise.
+    auto lane_again = [&]() {
+        uint32_t t = tid;
+        asm volatile("" : "+v"(t));
+        return t;
+    };
+    auto vidx = [&](int k, uint32_t t) {
+        const uint32_t v = v_begin + k * nt + t;
+        return FULL ? v : min(v, v_end - 1);
+    };
+    auto have = [&](int k, uint32_t t) { return FULL || v_begin + k * nt + t < v_end; };
+    // the address: a base that is the same for the whole workgroup (scalar registers) plus a
+    // lane offset, which for a full slice is the same for every k
+    auto at = [&](auto *base, int k, uint32_t t) {
+        using Byte = std::conditional_t<std::is_const<std::remove_pointer_t<decltype(base)>>::value, const char, char>;
+        const uint32_t offset = vidx(k, t) * (uint32_t)sizeof(u32x4);  // a unit is smaller than 4 GiB (host)
+        return reinterpret_cast<decltype(base)>(reinterpret_cast<Byte *>(base) + offset);
+    };
 #pragma unroll
-    for (int k = 0; k < K; k++) {
-        const uint32_t v = v_begin + k * nt + tid;
-        vidx[k] = FULL ? v : min(v, v_end - 1);
-        raw[k] = load_stream(xin + vidx[k]);
-    }
+    for (int k = 0; k < K; k++) raw[k] = load_stream(at(xin, k, tid));
     const uint32_t ch0 = (unit % p.groups) * p.ch_per_group;
     // optional per-(sample, channel) addend applied before the statistics (the reference's
     // chunkwise_add pass): the sum replaces the slice in registers, rounded to the storage
@@ -301,7 +321,7 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
         const T *cb = chunk + (size_t)(unit / p.groups) * (p.groups * p.ch_per_group);
 #pragma unroll
         for (int k = 0; k < K; k++) {
-            const float cv = Store<T>::load1(cb + ch0 + fast_div(vidx[k], p.hw_vec));
+            const float cv = Store<T>::load1(cb + ch0 + fast_div(vidx(k, tid), p.hw_vec));
             float f[EPV];
             Store<T>::unpack(raw[k], f);
 #pragma unroll
@@ -312,21 +332,28 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
     if (!FULL) {  // registers of lanes past the end of a ragged slice hold zeros from here on
 #pragma unroll
         for (int k = 0; k < K; k++) {
-            const bool have = v_begin + k * nt + tid < v_end;
+            const bool mine = have(k, tid);
 #pragma unroll
-            for (int i = 0; i < 4; i++) raw[k][i] = have ? raw[k][i] : 0u;
+            for (int i = 0; i < 4; i++) raw[k][i] = mine ? raw[k][i] : 0u;
         }
     }
-    // per-vector channel affine: fetched up front while the data is in flight when the
-    // registers allow it, otherwise just before use
-    constexpr bool kPrefetchAffine = K <= 6;
+    // per-vector channel affine.  Up to six vectors per lane: fetched into registers up front,
+    // while the data is in flight.  More: the group's gamma and beta go to LDS once (they are
+    // there after the barrier of the statistics) and the epilogue reads each vector's pair one
+    // vector ahead, so a lane's registers hold little besides its packed slice.
+    constexpr bool kPrefetchAffine = K <= kGnPrefetchAffineK;
     float ga[kPrefetchAffine ? K : 1], be[kPrefetchAffine ? K : 1];
     if (kPrefetchAffine) {
 #pragma unroll
         for (int k = 0; k < K; k++) {
-            const uint32_t c = ch0 + fast_div(vidx[k], p.hw_vec);
+            const uint32_t c = ch0 + fast_div(vidx(k, tid), p.hw_vec);
             ga[kPrefetchAffine ? k : 0] = gamma[c];
             be[kPrefetchAffine ? k : 0] = beta[c];
+        }
+    } else {
+        for (uint32_t c = tid; c < p.ch_per_group; c += nt) {  // ch_per_group <= kGnLdsChannels (host)
+            aff[c] = gamma[ch0 + c];
+            aff[kGnLdsChannels + c] = beta[ch0 + c];
         }
     }
 
@@ -364,6 +391,12 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
     // otherwise y = fma(x - mean, a, beta), which stays exact for |mean| >> sigma.
     auto epilogue = [&](auto fold_tag) {
         constexpr bool kFold = decltype(fold_tag)::value;
+        float g_next = 0.0f, b_next = 0.0f;
+        if (!kPrefetchAffine) {
+            const uint32_t c = fast_div(vidx(0, lane_again()), p.hw_vec);
+            g_next = aff[c];
+            b_next = aff[kGnLdsChannels + c];
+        }
 #pragma unroll
         for (int k = 0; k < K; k++) {
             float g_k, b_k;
@@ -371,9 +404,13 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
                 g_k = ga[kPrefetchAffine ? k : 0];
                 b_k = be[kPrefetchAffine ? k : 0];
             } else {
-                const uint32_t c = ch0 + fast_div(vidx[k], p.hw_vec);
-                g_k = gamma[c];
-                b_k = beta[c];
+                g_k = g_next;
+                b_k = b_next;
+                if (k + 1 < K) {  // the next vector's pair: its LDS latency passes under this vector's work
+                    const uint32_t c = fast_div(vidx(k + 1, lane_again()), p.hw_vec);
+                    g_next = aff[c];
+                    b_next = aff[kGnLdsChannels + c];
+                }
             }
             const float a = rstd * g_k;
             const float b_fold = fmaf(-mean, a, b_k);
@@ -386,7 +423,8 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
                 f[e] = SILU ? silu_f(t) : t;
             }
             const u32x4 packed = Store<T>::pack(f);
-            if (FULL || v_begin + k * nt + tid < v_end) store_stream(yout + vidx[k], packed);
+            const uint32_t t = lane_again();
+            if (have(k, t)) store_stream(at(yout, k, t), packed);
             // the scheduler must not start unpacking the next vectors before this one is stored:
             // eight elements are enough independent work, and the slice stays packed until used
             __builtin_amdgcn_sched_barrier(0);
@@ -409,16 +447,18 @@ __global__ __launch_bounds__(kGnMaxThreads, (K <= (sizeof(T) == 2 ? 5 : 4) ? 8 :
     __shared__ float red_b[kGnMaxThreads / kWave];
     __shared__ float red_c[kGnMaxThreads / kWave];
     __shared__ float stats[2];
+    __shared__ float aff[K <= kGnPrefetchAffineK ? 1 : 2 * kGnLdsChannels];  // gamma, beta of the group
     const uint32_t unit = blockIdx.x >> p.split_shift;
     const uint32_t slice = blockIdx.x & (p.split - 1);
     const uint32_t v_begin = slice * p.vec_per_slice;
     const uint32_t v_end = min(p.vec_per_unit, v_begin + p.vec_per_slice);
-    if (v_end - v_begin == K * blockDim.x)  // uniform over the workgroup
+    // uniform over the workgroup; the largest K is only launched on slices it fits exactly
+    if (K == kGnMaxK || v_end - v_begin == K * blockDim.x)
         gn_body<T, K, SILU, true>(x, chunk, y, gamma, beta, scratch, p, unit, slice, v_begin, v_end,
-                                  red_a, red_b, red_c, stats);
+                                  red_a, red_b, red_c, stats, aff);
     else
         gn_body<T, K, SILU, false>(x, chunk, y, gamma, beta, scratch, p, unit, slice, v_begin, v_end,
-                                   red_a, red_b, red_c, stats);
+                                   red_a, red_b, red_c, stats, aff);
 }
 
 // Any shape or alignment: one workgroup per unit, three passes over global memory with
@@ -609,7 +649,7 @@ __global__ __launch_bounds__(kGenericThreads) void gn_tokens_generic_kernel(
 // ---------------------------------------------------------------------------
 // Host: launch plan
 // ---------------------------------------------------------------------------
-const int kKValues[] = {1, 2, 3, 4, 5, 6, 8, 10, 12, 16};
+const int kKValues[] = {1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 20};
 
 inline int round_up_k(uint32_t k) {
     for (int v : kKValues)
@@ -623,30 +663,38 @@ struct GnPlan {
     int k;  // 0 = does not fit
 };
 
+// K for a slice of `vecs` vectors on `threads` lanes, 0 if there is none.  The largest K has
+// no code for a ragged slice: it takes equal slices that it fits exactly.
+int k_for(uint32_t vecs, uint32_t threads, uint32_t max_k, bool equal_slices) {
+    const int k = round_up_k((vecs + threads - 1) / threads);
+    if (k == 0 || (uint32_t)k > max_k) return 0;
+    if (k == kGnMaxK && !(equal_slices && vecs == (uint32_t)k * threads)) return 0;
+    return k;
+}
+
 // Threads and K for a slice of `vecs` vectors.  Measured on MI355X over every UNet shape
-// (workgroups of 256 ... 1024 lanes in steps of 64, 1 - 8 slices per unit): 512 lanes finish
-// soonest whenever the slice is at most 5 vectors per lane, even when the last wavefronts are
-// partly idle (a 320-vector unit: 2.95 us with 512 lanes, 3.18 us with exactly 320); larger
-// slices want 1024 lanes.  The tail of a slice that does not fill K * threads is masked.
-GnPlan plan_slice(uint32_t vecs, uint32_t split, uint32_t force_threads, uint32_t max_k, size_t blocks = 0) {
+// (workgroups of 256 ... 1024 lanes in steps of 64, 1 - 8 slices per unit): for a launch of
+// few workgroups 512 lanes finish soonest whenever the slice is at most 5 vectors per lane,
+// larger slices want 1024 lanes, and a small whole unit runs best with exactly one vector per
+// lane.  The tail of a slice that does not fill K * threads is masked.
+GnPlan plan_slice(uint32_t vecs, uint32_t split, uint32_t force_threads, uint32_t max_k, bool equal_slices,
+                  size_t blocks = 0) {
     GnPlan pl{split, 0, 0};
-    if (force_threads) {
+    if (force_threads && k_for(vecs, force_threads, max_k, equal_slices) != 0) {
         pl.threads = force_threads;
-    } else if (blocks >= 1024 && vecs >= 256) {
-        // Many workgroups per CU (large batches): throughput counts, not one workgroup's latency.
-        // Take the workgroup size that wastes the fewest lane slots, among those that keep a
-        // slice at five vectors per lane or fewer (64 registers, eight wavefronts per SIMD) when
-        // there is one.  Measured at batch 32, fp16: 2560-vector units 15.9 us with 512 lanes
-        // against 18.3 us with 1024; 1280-vector units 9.0 us with 256 lanes against 9.4 / 11.5 us.
-        uint32_t best_cost = 0xFFFFFFFFu;
-        for (uint32_t t : {1024u, 512u, 256u}) {
-            const int k = round_up_k((vecs + t - 1) / t);
-            if (k == 0 || (uint32_t)k > max_k) continue;
-            const uint32_t cost = (uint32_t)k * t + (k > 5 ? (1u << 24) : 0u);
-            if (cost < best_cost) {
-                best_cost = cost;
-                pl.threads = t;
-            }
+    } else if (blocks >= 2 * kChipCus && vecs >= 256) {
+        // Two or more workgroups per CU (large batches): throughput counts, not one workgroup's
+        // latency, and small workgroups that each hold many vectors per lane do best - more of
+        // them share a CU, in different phases (load / statistics / store), and a barrier joins
+        // four wavefronts, not sixteen.  Measured at batch 32 (1024 units), fp16, us per launch
+        // with 256 / 512 / 1024 lanes: 5120-vector units 30.1 / 33.6 / 31.8, 2560: 14.8 / 15.5 /
+        // 18.4, 1920: 12.0 / 13.1 / 15.4, 3840: 23.3 / 24.9 / 24.9; fp32 5120: 29.5 / 29.8 / 33.9.
+        // Batch 16 (512 units), 5120: 14.95 / 15.2 / 15.2; batch 12 is where 256 lanes lose
+        // (13.9 / 13.3 / 13.4) and the rules below take over.
+        for (uint32_t t : {256u, 512u, 768u, 1024u}) {
+            if (k_for(vecs, t, max_k, equal_slices) == 0) continue;
+            pl.threads = t;
+            break;
         }
         if (pl.threads == 0) pl.threads = kGnMaxThreads;
     } else if (vecs > 512u * 5u || (split > 1 && vecs >= 960))  // slices of a cut unit: 2 - 3 % faster
@@ -657,8 +705,7 @@ GnPlan plan_slice(uint32_t vecs, uint32_t split, uint32_t force_threads, uint32_
         pl.threads = 512;
     else
         pl.threads = ((vecs + kWave - 1) / kWave) * kWave;
-    pl.k = round_up_k((vecs + pl.threads - 1) / pl.threads);
-    if (pl.k == 0 || (uint32_t)pl.k > max_k) pl.k = 0;
+    pl.k = k_for(vecs, pl.threads, max_k, equal_slices);
     return pl;
 }
 
@@ -703,13 +750,13 @@ int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma
     if (units == 0 || unit_size == 0) return MSD_OK;
     if (units > 0x7FFFFFFFull || unit_size > 0x7FFFFFFFull) return MSD_ERR_INVALID_VALUE;
     if (fixed != nullptr && units > fixed->units) return MSD_ERR_SCRATCH_LIMIT;
-    if (!(aligned16(x) && aligned16(y) && hw % EPV == 0))
+    // (the register kernel addresses a unit with 32-bit byte offsets)
+    if (!(aligned16(x) && aligned16(y) && hw % EPV == 0) || unit_size * sizeof(T) >= (1ull << 32))
         return gn_generic<T>(silu, x, chunk, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
 
     const size_t vec_per_unit = unit_size / EPV;
-    // vectors per lane that stay in registers without spilling under the 1024-lane bound
-    constexpr uint32_t kMaxK = sizeof(T) == 4 ? 10 : kGnMaxK;
-    const size_t slice_cap = (size_t)kGnMaxThreads * kMaxK;  // vectors one workgroup can hold
+    constexpr uint32_t kMaxK = kGnMaxK;
+    const size_t slice_cap = (size_t)kGnMaxThreads * kGnMaxRaggedK;  // vectors one workgroup can hold
     // smallest power-of-two split whose slices fit in registers
     uint32_t split = 1;
     while ((size_t)split * slice_cap < vec_per_unit && split <= kGnMaxSplit) split *= 2;
@@ -733,11 +780,14 @@ int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma
             want = units >= 256 ? 1 : units >= 128 ? 2 : 4;
             if (units * 4 < 192 && unit_size >= 65536) want = 8;
         }
+        // Large batches of very long units (more than 10240 vectors): slices of up to 5120
+        // vectors on 256 lanes overlap better than whole units on 768 - 1024 lanes, the exchange
+        // disappears behind the other workgroups of the CU (batch 32, 15360-vector units: 90 us
+        // in four against 99 us whole)
+        if (units >= 2 * kChipCus && vec_per_unit > 10240)
+            while (vec_per_unit > (size_t)want * 5120 && want < kGnMaxSplit) want *= 2;
         while (units * want < 16 && want < kGnMaxSplit) want *= 2;  // very few units
         while (split < want && vec_per_unit >= (size_t)2 * split * 256) split *= 2;
-        // very long units (decoder-sized feature maps): keep a slice at 8 vectors per lane
-        // or fewer, which the 1024-lane register budget holds without spilling
-        while (split < kGnMaxSplit && (vec_per_unit + split - 1) / split > (size_t)kGnMaxThreads * 8) split *= 2;
     }
 
     GnParams p;
@@ -759,8 +809,9 @@ int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma
     if (tune_threads >= kWave && tune_threads <= kGnMaxThreads && tune_threads % kWave == 0 &&
         (size_t)tune_threads * kMaxK >= p.vec_per_slice)
         force_threads = (uint32_t)tune_threads;
-    const GnPlan pl = plan_slice(p.vec_per_slice, split, force_threads, kMaxK, units * split);
-    if (pl.k == 0)
+    const bool equal_slices = (size_t)p.vec_per_slice * split == vec_per_unit;
+    const GnPlan pl = plan_slice(p.vec_per_slice, split, force_threads, kMaxK, equal_slices, units * split);
+    if (pl.k == 0 || (pl.k > kGnPrefetchAffineK && cpg > kGnLdsChannels))
         return gn_generic<T>(silu, x, chunk, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
 
     GnScratch sc{nullptr, nullptr, nullptr, nullptr, nullptr, 0};
@@ -781,7 +832,8 @@ int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma
         case 8: gn_launch_k<T, 8>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
         case 10: gn_launch_k<T, 10>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
         case 12: gn_launch_k<T, 12>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
-        default: gn_launch_k<T, 16>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 16: gn_launch_k<T, 16>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        default: gn_launch_k<T, 20>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
     }
     return launch_status();
 }
@@ -807,7 +859,7 @@ template <typename T>
 int gn_tokens_dispatch(const void *xv, void *yv, const float *gamma, const float *beta, size_t batch,
                        size_t channels, size_t hw, size_t groups, float eps, hipStream_t stream) {
     constexpr int EPV = Store<T>::EPV;
-    constexpr uint32_t kMaxK = sizeof(T) == 4 ? 10 : kGnMaxK;
+    constexpr uint32_t kMaxK = sizeof(T) == 4 ? 10 : kGnMaxRaggedK;
     constexpr size_t kMaxLds = 60 * 1024;
     const T *x = static_cast<const T *>(xv);
     T *y = static_cast<T *>(yv);
@@ -868,7 +920,7 @@ int gn_tokens_dispatch(const void *xv, void *yv, const float *gamma, const float
     q.pitch = (uint32_t)(pvs * EPV + 16 / sizeof(T));
     q.combos = make_fast_div((uint32_t)(batch * split));
     const size_t lds_bytes = cpg * q.pitch * sizeof(T);
-    const GnPlan pl = plan_slice((uint32_t)nvec, split, 0, kMaxK);
+    const GnPlan pl = plan_slice((uint32_t)nvec, split, 0, kMaxK, false);
     if (pl.k == 0) return generic();
     GnScratch sc{nullptr, nullptr, nullptr, nullptr, nullptr, 0};
     if (split > 1) {

@@ -108,6 +108,63 @@ def test_groupnorm_every_split_factor(msd, orc, cuda, split, threads):
     assert msd.status() == 0
 
 
+@pytest.mark.parametrize("threads", [256, 320, 384, 448, 512, 576, 640, 768])
+def test_groupnorm_many_vectors_per_lane(msd, orc, cuda, threads):
+    """Small workgroups that hold 8 - 20 vectors per lane (what large batches run): exact and
+    ragged fits, gamma / beta through LDS, with and without SiLU, in place, with the ResBlock's
+    embedding add folded in, and one unit cut in two."""
+    import torch
+    lib = msd.load_library()
+    x = orc.normal((3, 320, 64, 64), seed=311 + threads, sigma=1.5, mean=0.4)
+    g, b = _affine(orc, 320, 311)
+    emb = orc.normal((3, 320), seed=312, sigma=0.5)
+    try:
+        assert lib.msd_set_tuning(msd.TUNE_GN_THREADS, threads) == 0
+        for half in (True, False):
+            _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half)
+            _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-6, False, half, inplace=True)
+            # a ragged fit: 9 channels of 64 x 48 per group
+            _run_groupnorm(msd, orc, cuda, x[:2, :288, :, :48].copy(), g[:288], b[:288], 32, 1e-5, True, half)
+            # chunkwise_add + GroupNorm in one launch against the two passes of the oracle
+            xin = orc.round_to_half(x) if half else x
+            ein = orc.round_to_half(emb) if half else emb
+            summed = xin + ein[:, :, None, None]
+            summed = orc.round_to_half(summed) if half else summed.astype(np.float32)
+            ref = orc.groupnorm(summed, g, b, 32, 1e-5, True)
+            got = msd.chunk_add_groupnorm(_to_dev(xin, cuda, half), _to_dev(ein, cuda, half), _to_dev(g, cuda),
+                                          _to_dev(b, cuda), 32, 1e-5, True).float().cpu().numpy()
+            if half:
+                assert_close_f16(got, ref, "chunk add groupnorm, %d lanes" % threads)
+            else:
+                assert_close_f32(got, ref, what="chunk add groupnorm f32, %d lanes" % threads)
+        assert lib.msd_set_tuning(msd.TUNE_GN_SPLIT, 2) == 0
+        _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, True)
+        _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, False)
+    finally:
+        lib.msd_set_tuning(msd.TUNE_GN_THREADS, 0)
+        lib.msd_set_tuning(msd.TUNE_GN_SPLIT, 0)
+    assert msd.status() == 0
+
+
+def test_groupnorm_large_batch_plan_and_wide_groups(msd, orc, cuda):
+    """What the launch plan picks by itself for many units (batch 17: 544 units, 256 lanes x 20
+    vectors), and a group of more channels than the LDS copy of gamma / beta holds (the general
+    kernel takes over)."""
+    lib = msd.load_library()
+    x = orc.normal((17, 320, 64, 64), seed=521, sigma=1.2, mean=-0.3)
+    g, b = _affine(orc, 320, 521)
+    _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, True)
+    _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, False)
+    wide = orc.normal((1, 32 * 1100, 16), seed=522, sigma=1.0)
+    gw, bw = _affine(orc, 32 * 1100, 522)
+    try:
+        assert lib.msd_set_tuning(msd.TUNE_GN_THREADS, 256) == 0  # 2200 vectors on 256 lanes: 10 per lane
+        _run_groupnorm(msd, orc, cuda, wide, gw, bw, 32, 1e-5, True, True)
+    finally:
+        lib.msd_set_tuning(msd.TUNE_GN_THREADS, 0)
+    assert msd.status() == 0
+
+
 @pytest.mark.parametrize("split", [2, 4, 16])
 def test_groupnorm_slice_that_stops_waiting_computes_its_siblings_statistics(msd, orc, cuda, split):
     """With a poll limit of one, nearly every workgroup gives up on its siblings at once and
