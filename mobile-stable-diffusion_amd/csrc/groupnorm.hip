@@ -159,16 +159,27 @@ __device__ __forceinline__ void gn_exchange(const GnScratch &scratch, const GnPa
         if (tid == 0) {
             stats[0] = total_mean;
             stats[1] = __builtin_amdgcn_rsqf(m2 * p.inv_count + p.eps);
-            // this slice has consumed its siblings' words; the last one closes the launch
-            const uint32_t old = __hip_atomic_fetch_add(scratch.done + unit, 1u, __ATOMIC_RELAXED,
-                                                        __HIP_MEMORY_SCOPE_AGENT);
-            if (old == p.split - 1) {
-                __hip_atomic_store(scratch.done + unit, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(scratch.epoch + unit, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
         }
     }
     __syncthreads();
+}
+
+// This slice has consumed its siblings' words: it counts itself done.  Called by lane 0 of the
+// workgroup after the barrier that ends gn_exchange, so that no wavefront waits for the
+// counter's old value, which comes back a memory round trip later; gn_exchange_close uses it
+// at the end of the kernel.
+__device__ __forceinline__ uint32_t gn_exchange_arrive(const GnScratch &scratch, uint32_t unit) {
+    return __hip_atomic_fetch_add(scratch.done + unit, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The last slice to arrive closes the launch: the counter goes back to zero and the unit's
+// launch count advances (both visible to the next launch, which starts after this kernel).
+__device__ __forceinline__ void gn_exchange_close(const GnScratch &scratch, const GnParams &p, uint32_t unit,
+                                                  uint32_t epoch, uint32_t arrived_before) {
+    if (arrived_before == p.split - 1) {
+        __hip_atomic_store(scratch.done + unit, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(scratch.epoch + unit, epoch + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 }
 
 // Sum and sum of squares of a packed vector, accumulated in float32.  Half storage uses
@@ -361,6 +372,7 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
     gn_slice_stats<T, K, FULL>(raw, v_end - v_begin, red_a, red_b, red_c, slice_mean, slice_m2);
 
     float mean, rstd;
+    uint32_t arrived_before = 0;
     if (p.split == 1) {
         mean = slice_mean;
         rstd = __builtin_amdgcn_rsqf(slice_m2 * p.inv_count + p.eps);
@@ -383,6 +395,7 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
         gn_exchange<T>(scratch, p, unit, slice, epoch, slice_mean, slice_m2, stats, read);
         mean = stats[0];
         rstd = stats[1];
+        if (tid == 0) arrived_before = gn_exchange_arrive(scratch, unit);
     }
 
     // ---- normalise from registers, per-channel affine, optional SiLU.  When the unit's mean is
@@ -434,6 +447,7 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
         epilogue(std::true_type{});
     else
         epilogue(std::false_type{});
+    if (p.split > 1 && tid == 0) gn_exchange_close(scratch, p, unit, epoch, arrived_before);
 }
 
 // Up to five vectors per lane (four for float storage) the kernel fits 64 registers: eight
@@ -594,6 +608,9 @@ __global__ __launch_bounds__(kGnMaxThreads) void gn_tokens_kernel(
         }
     }
     __syncthreads();
+    // the slice counts itself done here, behind the last barrier: nothing waits for the answer
+    uint32_t arrived_before = 0;
+    if (p.split > 1 && tid == 0) arrived_before = gn_exchange_arrive(scratch, unit);
 
     // ---- token-major store: for each position of the slice one run of ch_per_group values
     const uint32_t rows = pvs * EPV;                         // positions in the slice
@@ -615,6 +632,7 @@ __global__ __launch_bounds__(kGnMaxThreads) void gn_tokens_kernel(
         }
         out[(size_t)r * row_stride + c] = w;
     }
+    if (p.split > 1 && tid == 0) gn_exchange_close(scratch, p, unit, epoch, arrived_before);
 }
 
 // Any shape: one workgroup per unit, three passes, element-wise scattered stores.

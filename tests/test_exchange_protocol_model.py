@@ -8,8 +8,9 @@ What the kernel does per slice, and what the model replays one memory operation 
   3. lane l polls slice l's two words until both carry the tag, at most `spin_limit` times;
      a sibling that has not published by then is computed from the sibling's part of the INPUT
      (two passes), after which its words are read once more and win if they have arrived
-  4. merge all slices (Chan), then fetch_add(done); the last slice stores done = 0, epoch = tag
+  4. merge all slices (Chan), then fetch_add(done) (its old value is used in step 6)
   5. only now store the output over its own part (the call may be in place)
+  6. the slice whose fetch_add returned split - 1 stores done = 0, epoch = tag
 
 All of it is relaxed atomics: stores become visible to the other slices after arbitrary delays
 and in any order across addresses.  Two things the protocol leans on are modelled as facts of
@@ -123,13 +124,13 @@ class Launch:
         old = u.done                          # 4. fetch_add is atomic at memory: immediate
         u.done = old + 1
         yield
-        if old == self.split - 1:
+        self.store(s, "output", s, True)      # 5.
+        yield
+        if old == self.split - 1:             # 6.
             self.store(s, "done", 0, 0)
             yield
             self.store(s, "epoch", 0, tag)
             yield
-        self.store(s, "output", s, True)      # 5.
-        yield
         self.finished[s] = True
 
     def run(self, starve=None):
