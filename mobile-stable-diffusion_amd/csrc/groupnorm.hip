@@ -6,14 +6,16 @@
 // the tensor is read from HBM once and written once.
 //
 //   1. every lane issues all its loads (K vectors) before the first use;
-//   2. slice mean, then slice M2 = sum (x - slice mean)^2, both from registers
-//      (DPP wavefront reduction, one LDS slot per wavefront);
+//   2. slice mean and M2 = sum (x - slice mean)^2 from one pass of sum and sum of squares
+//      over the packed registers (DPP wavefront reduction, one LDS slot per wavefront), with
+//      a second, centred pass when the mean is large against the spread;
 //   3. split > 1: slices publish (mean, M2) as two tagged 64-bit words, poll
 //      their siblings' words, and merge with Chan's formula.  The tag is the
 //      unit's launch count, read at kernel start; the last slice to finish
 //      advances it, so nothing is reset between launches and a replayed graph
 //      works.  All traffic is relaxed agent-scope atomics: no cache flushes.
-//   4. y = fma(x - mean, rstd * gamma[c], beta[c]), optional SiLU, packed store.
+//   4. y = fma(x - mean, rstd * gamma[c], beta[c]) (the mean folded into the offset when it
+//      is small), optional SiLU, packed store.
 //
 // Workgroups of one unit have adjacent block ids, so a waiter's siblings are
 // normally dispatched together with it.  Nothing depends on that: a wait is
@@ -799,12 +801,12 @@ int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma
             vec_per_unit >= (size_t)forced * kWave)
             split = forced;
     } else if (can_split) {
-        // A workgroup's time grows with its slice (about 0.13 us per 1024 elements on MI355X,
-        // it is latency- and ALU-bound, not bandwidth-bound) while the exchange between the
-        // slices of a unit costs 1.3 - 2.5 us, so units up to 24 Ki elements stay whole and
-        // larger ones are cut in four; eight when that still leaves most of the chip idle.
+        // A workgroup's time grows with its slice (one CU loads, reduces and normalises it) while
+        // the exchange between the slices of a unit costs 1.3 - 1.9 us (two round trips through
+        // the memory-side coherence point), so units up to 24 Ki elements stay whole and larger
+        // ones are cut in two or four; eight when that still leaves most of the chip idle.
         // With 256 or more units every CU has one of its own and cutting only adds the exchange
-        // (batch 8, 320 channels at 64x64: 9.9 us whole against 13.8 us in four).
+        // (batch 8, 320 channels at 64x64: 9.0 us whole against 10.5 us in two).
         uint32_t want = 1;
         if (unit_size > 24576) {
             // (up to 32 Ki elements two slices are enough: 960 channels at 32 x 32, 5.40 us in two
