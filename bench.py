@@ -266,6 +266,12 @@ def _rotating_launch_us(torch, msd, stream, launch, xs, ys, warm=20, budget=2000
         return event_time_ms(torch, replay, reps) * 1e3 / (reps * copies)
 
 
+def _gn_plan_text(msd, batch, channels, hw, elt):
+    """'slices per unit x lanes x vectors per lane' of the GroupNorm launch for this shape."""
+    split, threads, k = msd.groupnorm_plan(batch, channels, hw, 32, msd.DTYPE_F16 if elt == 2 else msd.DTYPE_F32)
+    return "general kernel" if split == 0 else "%d x %d lanes x %d vectors" % (split, threads, k)
+
+
 def _kernel_case(torch, msd, dev, kind, p, dt, batch):
     """Buffers, launch closure and byte counts for one row of the per-kernel tables."""
     import ctypes
@@ -340,6 +346,8 @@ def shape_table(torch, msd, dev, stream):
             row["pct_of_copy_rate"] = round(100.0 * cus / us, 1)
         if cfg in ("cfg1", "cfg4"):
             row["note"] = "launch-bound: %.2f us at 8 TB/s" % (case["bytes"] / HBM_PEAK_GBS / 1e3)
+        if kind == "groupnorm_silu":
+            row["plan"] = _gn_plan_text(msd, batch, p["c"], p["hw"], case["elt"])
         rows.append(row)
         del case
         torch.cuda.empty_cache()
@@ -672,6 +680,8 @@ def large_batch_table(torch, msd, dev, stream):
             cus = measure(copy_body, copies)
             row["copy_us"] = round(cus, 2)
             row["pct_of_copy_rate"] = round(100 * cus / us, 1)
+        if kind == "groupnorm_silu":
+            row["plan"] = _gn_plan_text(msd, B, p["c"], p["hw"], 2)
         rows.append(row)
         del xs, ys
         torch.cuda.empty_cache()

@@ -121,6 +121,17 @@ int msd_groupnorm_noalloc(const void *x, void *y, const float *gamma, const floa
                           int fuse_silu, int dtype, void *stream);
 
 /*
+ * The launch msd_groupnorm (noalloc != 0: msd_groupnorm_noalloc) makes for this shape on 16-byte
+ * aligned tensors, under the tuning knobs as they are set: *split workgroups per (sample, group),
+ * *threads lanes each, *vectors_per_lane 16-byte vectors held per lane.  *split = 0 (the others
+ * too) means the general kernel: one 256-lane workgroup per (sample, group), nothing held in
+ * registers.  Host arithmetic only: needs no GPU and launches nothing.  For diagnostics, tests and
+ * benchmark tables.  No counterpart in the reference (its geometry is fixed, M/nn/GroupNorm.cpp:105-128).
+ */
+int msd_groupnorm_plan(size_t batch, size_t channels, size_t hw, size_t groups, int dtype, int noalloc,
+                       int *split, int *threads, int *vectors_per_lane);
+
+/*
  * GroupNorm whose result is stored token-major: x is [batch, channels, hw], y is
  * [batch, hw, channels], y[b, p, c] = GroupNorm(x)[b, c, p].  Replaces GroupNorm::forward
  * followed by the permute3D_0_2_1 enqueue of SpatialTransformer::forward

@@ -24,7 +24,7 @@ ERR_SCRATCH_LIMIT = -2
 # every symbol include/msd_hip.h declares
 C_ABI_SYMBOLS = (
     "msd_version", "msd_error_string", "msd_init", "msd_release", "msd_shutdown", "msd_status",
-    "msd_gn_fallbacks", "msd_set_tuning", "msd_groupnorm", "msd_groupnorm_noalloc", "msd_layernorm", "msd_geglu",
+    "msd_gn_fallbacks", "msd_set_tuning", "msd_groupnorm", "msd_groupnorm_noalloc", "msd_groupnorm_plan", "msd_layernorm", "msd_geglu",
     "msd_silu", "msd_gelu", "msd_quick_gelu", "msd_timestep_embedding", "msd_ddim_timesteps",
     "msd_elemwise_add", "msd_chunkwise_add", "msd_chunk_add_groupnorm", "msd_add_layernorm", "msd_copy",
     "msd_groupnorm_tokens", "msd_permute_0_2_1",
@@ -62,6 +62,7 @@ def load_library(path=None):
     lib.msd_set_tuning.argtypes = [it, it]
     lib.msd_groupnorm.argtypes = [vp, vp, vp, vp, sz, sz, sz, sz, fl, it, it, vp]
     lib.msd_groupnorm_noalloc.argtypes = [vp, vp, vp, vp, sz, sz, sz, sz, fl, it, it, vp]
+    lib.msd_groupnorm_plan.argtypes = [sz, sz, sz, sz, it, it] + [ctypes.POINTER(ctypes.c_int)] * 3
     lib.msd_layernorm.argtypes = [vp, vp, vp, vp, sz, sz, fl, it, vp]
     lib.msd_geglu.argtypes = [vp, vp, sz, sz, it, vp]
     lib.msd_copy.argtypes = [vp, vp, sz, vp]
@@ -160,6 +161,15 @@ def groupnorm(x, gamma, beta, groups, eps=1e-5, fuse_silu=False, out=None, noall
              _affine(beta, channels, x, "beta"), batch, channels, hw, groups, eps, int(fuse_silu),
              _dtype_code(x), _stream()))
     return out
+
+
+def groupnorm_plan(batch, channels, hw, groups=32, dtype_code=DTYPE_F16, noalloc=False):
+    """(split, threads, vectors per lane) of the launch msd_groupnorm makes for this shape;
+    (0, 0, 0) = the general kernel.  Host arithmetic, no GPU needed."""
+    out = [ctypes.c_int(0) for _ in range(3)]
+    check(load_library().msd_groupnorm_plan(batch, channels, hw, groups, dtype_code, int(noalloc),
+                                            *[ctypes.byref(o) for o in out]))
+    return tuple(o.value for o in out)
 
 
 def groupnorm_tokens(x, gamma, beta, groups, eps=1e-6):

@@ -250,6 +250,23 @@ int msd_groupnorm(const void *x, void *y, const float *gamma, const float *beta,
                            dtype, nullptr, stream);
 }
 
+int msd_groupnorm_plan(size_t batch, size_t channels, size_t hw, size_t groups, int dtype, int noalloc,
+                       int *split, int *threads, int *vectors_per_lane) {
+    if (!split || !threads || !vectors_per_lane) return MSD_ERR_INVALID_VALUE;
+    if (groups == 0 || channels == 0 || channels % groups != 0) return MSD_ERR_INVALID_VALUE;
+    if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
+    if (batch * groups > 0x7FFFFFFFull || (channels / groups) * hw > 0x7FFFFFFFull) return MSD_ERR_INVALID_VALUE;
+    if (noalloc && batch * groups > kStaticUnits) return MSD_ERR_SCRATCH_LIMIT;
+    GnDecision d{0, 0, 0, 0};
+    if (batch * hw != 0)
+        d = gn_decide(dtype == MSD_DTYPE_F32 ? 4 : 2, batch, channels, hw, groups, true,
+                      noalloc ? (size_t)kStaticUnits : (size_t)kGnMaxUnits);
+    *split = (int)d.split;
+    *threads = (int)d.threads;
+    *vectors_per_lane = (int)d.k;
+    return MSD_OK;
+}
+
 int msd_groupnorm_noalloc(const void *x, void *y, const float *gamma, const float *beta, size_t batch,
                           size_t channels, size_t hw, size_t groups, float eps, int fuse_silu, int dtype,
                           void *stream) {

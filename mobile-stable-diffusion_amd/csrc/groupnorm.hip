@@ -727,7 +727,9 @@ GnPlan plan_slice(uint32_t vecs, uint32_t split, uint32_t force_threads, uint32_
             break;
         }
         if (pl.threads == 0) pl.threads = kGnMaxThreads;
-    } else if (uint32_t exact = exact_fit_threads(vecs)) {
+    } else if (uint32_t exact = (split == 1 && vecs == 1280) ? 0u : exact_fit_threads(vecs)) {
+        // (a whole unit of 1280 vectors is the exception: 3.55 us on 512 lanes with a masked tail
+        // against 3.62 us on 640 x 2)
         pl.threads = exact;
     } else if (vecs > 512u * 5u || (split > 1 && vecs >= 960))  // slices of a cut unit: 2 - 3 % faster
         pl.threads = kGnMaxThreads;
@@ -765,36 +767,30 @@ int gn_generic(bool silu, const T *x, const T *chunk, T *y, const float *gamma, 
 
 }  // namespace
 
-template <typename T>
-int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma, const float *beta,
-                size_t batch, size_t channels, size_t hw, size_t groups, float eps, bool silu,
-                const GnScratch *fixed, hipStream_t stream) {
-    constexpr int EPV = Store<T>::EPV;
+// What a GroupNorm launch looks like for a shape: split == 0 means the general kernel (one
+// workgroup per unit, any alignment); otherwise `split` workgroups of `threads` lanes per unit,
+// each holding its slice as `k` vectors per lane.  `elt` = bytes per element, `max_units` = units
+// the exchange scratch has room for.  Reads the tuning knobs.
+GnDecision gn_decide(size_t elt, size_t batch, size_t channels, size_t hw, size_t groups, bool aligned,
+                     size_t max_units) {
+    GnDecision d{0, 0, 0, 0};
+    const size_t epv = 16 / elt;
     const int tune_split = g_tuning.gn_split.load(std::memory_order_relaxed);
     const int tune_threads = g_tuning.gn_threads.load(std::memory_order_relaxed);
-    const int tune_spin = g_tuning.gn_spin_limit.load(std::memory_order_relaxed);
-    const T *x = static_cast<const T *>(xv);
-    const T *chunk = static_cast<const T *>(chunkv);
-    T *y = static_cast<T *>(yv);
     const size_t cpg = channels / groups;
     const size_t unit_size = cpg * hw;
     const size_t units = batch * groups;
-    if (units == 0 || unit_size == 0) return MSD_OK;
-    if (units > 0x7FFFFFFFull || unit_size > 0x7FFFFFFFull) return MSD_ERR_INVALID_VALUE;
-    if (fixed != nullptr && units > fixed->units) return MSD_ERR_SCRATCH_LIMIT;
     // (the register kernel addresses a unit with 32-bit byte offsets)
-    if (!(aligned16(x) && aligned16(y) && hw % EPV == 0) || unit_size * sizeof(T) >= (1ull << 32))
-        return gn_generic<T>(silu, x, chunk, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
+    if (!aligned || hw % epv != 0 || unit_size * elt >= (1ull << 32)) return d;
 
-    const size_t vec_per_unit = unit_size / EPV;
+    const size_t vec_per_unit = unit_size / epv;
     constexpr uint32_t kMaxK = kGnMaxK;
     const size_t slice_cap = (size_t)kGnMaxThreads * kGnMaxRaggedK;  // vectors one workgroup can hold
     // smallest power-of-two split whose slices fit in registers
     uint32_t split = 1;
     while ((size_t)split * slice_cap < vec_per_unit && split <= kGnMaxSplit) split *= 2;
-    const bool can_split = units <= (fixed != nullptr ? fixed->units : kGnMaxUnits);
-    if (split > kGnMaxSplit || (split > 1 && !can_split))
-        return gn_generic<T>(silu, x, chunk, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
+    const bool can_split = units <= max_units;
+    if (split > kGnMaxSplit || (split > 1 && !can_split)) return d;
     if (tune_split > 0) {
         uint32_t forced = (uint32_t)tune_split;
         if (forced > split && can_split && (forced & (forced - 1)) == 0 && forced <= kGnMaxSplit &&
@@ -824,9 +820,48 @@ int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma
         while (split < want && vec_per_unit >= (size_t)2 * split * 256) split *= 2;
     }
 
+    const size_t vec_per_slice = (vec_per_unit + split - 1) / split;
+    // every slice must own at least one vector (ceil division can starve the last ones)
+    if (vec_per_slice * (split - 1) >= vec_per_unit) return d;
+
+    uint32_t force_threads = 0;
+    if (tune_threads >= kWave && tune_threads <= kGnMaxThreads && tune_threads % kWave == 0 &&
+        (size_t)tune_threads * kMaxK >= vec_per_slice)
+        force_threads = (uint32_t)tune_threads;
+    const bool equal_slices = vec_per_slice * split == vec_per_unit;
+    const GnPlan pl = plan_slice((uint32_t)vec_per_slice, split, force_threads, kMaxK, equal_slices, units * split);
+    if (pl.k == 0 || (pl.k > kGnPrefetchAffineK && cpg > kGnLdsChannels)) return d;
+    d.split = split;
+    d.threads = pl.threads;
+    d.k = (uint32_t)pl.k;
+    d.vec_per_slice = (uint32_t)vec_per_slice;
+    return d;
+}
+
+template <typename T>
+int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma, const float *beta,
+                size_t batch, size_t channels, size_t hw, size_t groups, float eps, bool silu,
+                const GnScratch *fixed, hipStream_t stream) {
+    constexpr int EPV = Store<T>::EPV;
+    const int tune_spin = g_tuning.gn_spin_limit.load(std::memory_order_relaxed);
+    const T *x = static_cast<const T *>(xv);
+    const T *chunk = static_cast<const T *>(chunkv);
+    T *y = static_cast<T *>(yv);
+    const size_t cpg = channels / groups;
+    const size_t unit_size = cpg * hw;
+    const size_t units = batch * groups;
+    if (units == 0 || unit_size == 0) return MSD_OK;
+    if (units > 0x7FFFFFFFull || unit_size > 0x7FFFFFFFull) return MSD_ERR_INVALID_VALUE;
+    if (fixed != nullptr && units > fixed->units) return MSD_ERR_SCRATCH_LIMIT;
+    const GnDecision d = gn_decide(sizeof(T), batch, channels, hw, groups, aligned16(x) && aligned16(y),
+                                   fixed != nullptr ? fixed->units : kGnMaxUnits);
+    if (d.split == 0)
+        return gn_generic<T>(silu, x, chunk, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
+
+    const uint32_t split = d.split;
     GnParams p;
-    p.vec_per_unit = (uint32_t)vec_per_unit;
-    p.vec_per_slice = (uint32_t)((vec_per_unit + split - 1) / split);
+    p.vec_per_unit = (uint32_t)(unit_size / EPV);
+    p.vec_per_slice = d.vec_per_slice;
     p.split = split;
     p.split_shift = (uint32_t)__builtin_ctz(split);
     p.groups = (uint32_t)groups;
@@ -835,18 +870,6 @@ int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma
     p.eps = eps;
     p.inv_count = 1.0f / (float)unit_size;
     p.spin_limit = tune_spin > 0 ? (uint32_t)tune_spin : kGnSpinLimit;
-    // every slice must own at least one vector (ceil division can starve the last ones)
-    if ((size_t)p.vec_per_slice * (split - 1) >= vec_per_unit)
-        return gn_generic<T>(silu, x, chunk, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
-
-    uint32_t force_threads = 0;
-    if (tune_threads >= kWave && tune_threads <= kGnMaxThreads && tune_threads % kWave == 0 &&
-        (size_t)tune_threads * kMaxK >= p.vec_per_slice)
-        force_threads = (uint32_t)tune_threads;
-    const bool equal_slices = (size_t)p.vec_per_slice * split == vec_per_unit;
-    const GnPlan pl = plan_slice(p.vec_per_slice, split, force_threads, kMaxK, equal_slices, units * split);
-    if (pl.k == 0 || (pl.k > kGnPrefetchAffineK && cpg > kGnLdsChannels))
-        return gn_generic<T>(silu, x, chunk, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
 
     GnScratch sc{nullptr, nullptr, nullptr, nullptr, nullptr, 0};
     if (fixed != nullptr) {
@@ -856,18 +879,20 @@ int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma
         if (err != hipSuccess) return (int)err;
     }
     const uint32_t blocks = (uint32_t)(units * split);
-    switch (pl.k) {
-        case 1: gn_launch_k<T, 1>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
-        case 2: gn_launch_k<T, 2>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
-        case 3: gn_launch_k<T, 3>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
-        case 4: gn_launch_k<T, 4>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
-        case 5: gn_launch_k<T, 5>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
-        case 6: gn_launch_k<T, 6>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
-        case 8: gn_launch_k<T, 8>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
-        case 10: gn_launch_k<T, 10>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
-        case 12: gn_launch_k<T, 12>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
-        case 16: gn_launch_k<T, 16>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
-        default: gn_launch_k<T, 20>(silu, blocks, pl.threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+    const uint32_t threads = d.threads;
+    switch (d.k) {
+        case 1: gn_launch_k<T, 1>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 2: gn_launch_k<T, 2>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 3: gn_launch_k<T, 3>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 4: gn_launch_k<T, 4>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 5: gn_launch_k<T, 5>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 6: gn_launch_k<T, 6>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 8: gn_launch_k<T, 8>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 10: gn_launch_k<T, 10>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 12: gn_launch_k<T, 12>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 16: gn_launch_k<T, 16>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 20: gn_launch_k<T, 20>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        default: return MSD_ERR_INVALID_VALUE;  // not a K the kernels are built for: a planning error
     }
     return launch_status();
 }

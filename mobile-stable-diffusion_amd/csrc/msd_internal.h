@@ -45,6 +45,18 @@ struct Tuning {
 };
 extern Tuning g_tuning;
 
+// The launch msd_groupnorm makes for a shape (see gn_decide in groupnorm.hip): split == 0 is the
+// general kernel, otherwise split workgroups of `threads` lanes per (sample, group), k 16-byte
+// vectors per lane, vec_per_slice vectors per workgroup.
+struct GnDecision {
+    uint32_t split;
+    uint32_t threads;
+    uint32_t k;
+    uint32_t vec_per_slice;
+};
+GnDecision gn_decide(size_t elt, size_t batch, size_t channels, size_t hw, size_t groups, bool aligned,
+                     size_t max_units);
+
 // ---- per-dtype dispatchers (T = float or __half), defined in the kernel files ----
 // fixed: scratch to use instead of the stream's own (units beyond its capacity are refused)
 template <typename T>

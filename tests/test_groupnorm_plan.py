@@ -1,0 +1,95 @@
+"""The launch plan of msd_groupnorm, checked on the CPU through msd_groupnorm_plan (host arithmetic).
+
+A kernel that does not match its launch faults the GPU, so what the planner may hand to the
+register kernel is pinned here: the vectors-per-lane values the kernels are built for, workgroup
+sizes in whole wavefronts, slices that fit their workgroup and own at least one vector, the largest
+vectors-per-lane value only on exact fits, power-of-two slice counts within the exchange scratch.
+The reference has no counterpart: its geometry is fixed (M/nn/GroupNorm.cpp:105-128)."""
+import importlib
+import random
+
+import pytest
+
+msd = importlib.import_module("mobile-stable-diffusion_amd")
+
+K_VALUES = {1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 20}
+MAX_SPLIT, MAX_UNITS, STATIC_UNITS = 64, 8192, 1024
+
+
+def _check(batch, channels, hw, groups, code, noalloc=False):
+    split, threads, k = msd.groupnorm_plan(batch, channels, hw, groups, code, noalloc)
+    elt = 4 if code == msd.DTYPE_F32 else 2
+    epv = 16 // elt
+    unit = channels // groups * hw
+    if split == 0:
+        assert threads == 0 and k == 0
+        return split, threads, k
+    assert hw % epv == 0 and unit * elt < 2 ** 32          # what the register kernel assumes
+    vecs = unit // epv
+    assert split & (split - 1) == 0 and 1 <= split <= MAX_SPLIT
+    if split > 1:
+        assert batch * groups <= (STATIC_UNITS if noalloc else MAX_UNITS)
+    assert threads % 64 == 0 and 64 <= threads <= 1024
+    assert k in K_VALUES
+    per_slice = -(-vecs // split)
+    assert per_slice * (split - 1) < vecs                  # the last slice owns at least one vector
+    assert k * threads >= per_slice                        # a slice fits its workgroup's registers
+    assert (k - 1) * threads < per_slice or k == min(v for v in K_VALUES if v * threads >= per_slice)
+    if k == 20:                                            # no masked code for the largest K
+        assert per_slice * split == vecs and per_slice == 20 * threads
+    if k > 6:                                              # gamma / beta of the group go through LDS
+        assert channels // groups <= 1024
+    return split, threads, k
+
+
+def test_plans_of_the_unet_shapes_at_batch_2_and_32():
+    f16, f32 = msd.DTYPE_F16, msd.DTYPE_F32
+    expected = {
+        (2, 320, 4096, f16): (4, 640, 2), (2, 640, 1024, f16): (1, 512, 5), (2, 1280, 256, f16): (1, 512, 3),
+        (2, 1280, 64, f16): (1, 320, 1), (2, 960, 1024, f16): (2, 960, 2), (2, 1920, 256, f16): (1, 960, 2),
+        (1, 320, 4096, f32): (4, 1024, 3),
+        (32, 320, 4096, f16): (1, 256, 20), (32, 640, 1024, f16): (1, 256, 10), (32, 1280, 256, f16): (1, 256, 5),
+        (8, 320, 4096, f16): (1, 1024, 5), (32, 960, 4096, f16): (4, 256, 16),
+    }
+    for (batch, channels, hw, code), want in expected.items():
+        assert _check(batch, channels, hw, 32, code) == want, (batch, channels, hw, code)
+
+
+def test_shapes_the_register_kernel_cannot_take_go_to_the_general_kernel():
+    assert msd.groupnorm_plan(2, 320, 4090, 32, msd.DTYPE_F16) == (0, 0, 0)      # hw not in whole vectors
+    assert msd.groupnorm_plan(2, 320, 4094, 32, msd.DTYPE_F32) == (0, 0, 0)
+    assert msd.groupnorm_plan(1, 32 * 1100, 32, 32, msd.DTYPE_F16)[2] <= 6         # wide groups: no LDS affine
+    assert msd.groupnorm_plan(0, 320, 4096, 32, msd.DTYPE_F16) == (0, 0, 0)        # nothing to do
+    lib = msd.load_library()
+    import ctypes
+    o = [ctypes.c_int(7) for _ in range(3)]
+    refs = [ctypes.byref(v) for v in o]
+    assert lib.msd_groupnorm_plan(2, 320, 4096, 0, msd.DTYPE_F16, 0, *refs) == 1   # no groups
+    assert lib.msd_groupnorm_plan(2, 321, 4096, 32, msd.DTYPE_F16, 0, *refs) == 1  # channels % groups
+    assert lib.msd_groupnorm_plan(2, 320, 4096, 32, 5, 0, *refs) == 1              # unknown dtype
+    assert lib.msd_groupnorm_plan(2, 320, 4096, 32, msd.DTYPE_F16, 0, None, None, None) == 1
+    assert lib.msd_groupnorm_plan(33, 320, 4096, 32, msd.DTYPE_F16, 1, *refs) == -2  # beyond the fixed scratch
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_shapes_always_get_a_launch_that_fits(seed):
+    rng = random.Random(seed)
+    lib = msd.load_library()
+    knobs = [(0, 0)] + [(rng.choice([0, 1, 2, 4, 8, 16, 32, 64]), rng.choice([0, 64, 128, 256, 320, 512, 640, 768, 1024]))
+                        for _ in range(3)]
+    try:
+        for split_knob, threads_knob in knobs:
+            assert lib.msd_set_tuning(msd.TUNE_GN_SPLIT, split_knob) == 0
+            assert lib.msd_set_tuning(msd.TUNE_GN_THREADS, threads_knob) == 0
+            for _ in range(1500):
+                groups = rng.choice([1, 2, 8, 32, 32, 32, 64])
+                cpg = rng.choice([1, 2, 3, 5, 10, 20, 30, 40, 60, 80, 128, 1100])
+                hw = rng.choice([8, 16, 24, 64, 72, 256, 1000, 1024, 4096, 4104, 16384, 65536, 262144])
+                batch = rng.choice([1, 2, 2, 3, 8, 16, 32, 64, 300])
+                code = rng.choice([msd.DTYPE_F16, msd.DTYPE_F32])
+                if cpg * hw > 0x7FFFFFFF or batch * groups > 0x7FFFFFFF:
+                    continue
+                _check(batch, groups * cpg, hw, groups, code, noalloc=batch * groups <= STATIC_UNITS and rng.random() < 0.3)
+    finally:
+        lib.msd_set_tuning(msd.TUNE_GN_SPLIT, 0)
+        lib.msd_set_tuning(msd.TUNE_GN_THREADS, 0)
