@@ -275,8 +275,8 @@ def test_softmax_full_size_rows_sum_to_one(msd, cuda):
     assert float((sums - 1.0).abs().max()) < 2e-2  # 4096 values rounded to fp16 each
     assert float(x.min()) >= 0.0 and float(x.max()) <= 1.0
     e = np.exp(keep.astype(np.float64))
-    np.testing.assert_allclose(x[:64].float().cpu().numpy(), e / e.sum(axis=-1, keepdims=True),
-                               atol=2e-3, rtol=1e-3)
+    assert_close_f16(x[:64].float().cpu().numpy(), e / e.sum(axis=-1, keepdims=True), "softmax 65536x4096, 64 rows",
+                     rel_floor=0.0)
 
 
 # ----------------------------------------------------------------- DDIM
