@@ -355,16 +355,23 @@ def shape_table(torch, msd, dev, stream):
 
 
 def launch_floor_us(torch, msd, dev, stream):
-    """µs per launch of a chain of 16-byte copies replayed as a graph: what one more kernel in
-    a captured step costs when it moves nothing."""
+    """(µs per launch, µs per graph launch): what one more kernel in a captured step costs when
+    it moves nothing, and what launching a graph costs whatever it holds.  Chains of 128 and 512
+    16-byte copies are replayed as graphs; the first figure is the slope between the two chain
+    lengths, the second the remainder of the shorter chain."""
     import ctypes
     vp = ctypes.c_void_p
     lib = msd.load_library()
-    xs = [torch.zeros(4, device=dev) for _ in range(64)]
-    ys = [torch.zeros(4, device=dev) for _ in range(64)]
-    return _rotating_launch_us(torch, msd, stream,
-                               lambda x, y, sp: lib.msd_copy(vp(x.data_ptr()), vp(y.data_ptr()), 16, sp), xs, ys,
-                               budget=20000)
+    xs = [torch.zeros(4, device=dev) for _ in range(512)]
+    ys = [torch.zeros(4, device=dev) for _ in range(512)]
+
+    def chain(nodes):
+        return nodes * _rotating_launch_us(torch, msd, stream,
+                                           lambda x, y, sp: lib.msd_copy(vp(x.data_ptr()), vp(y.data_ptr()), 16, sp),
+                                           xs[:nodes], ys[:nodes], budget=40000)
+    short, long_ = chain(128), chain(512)
+    per_launch = (long_ - short) / 384.0
+    return per_launch, max(0.0, short - 128 * per_launch)
 
 
 def gn_split_table(torch, msd, dev, stream):
@@ -1023,7 +1030,9 @@ def main():
         "roofline_families": roofline_families,
         "kernel_families": families,
     }
-    out["config"]["launch_floor_us"] = round(launch_floor_us(torch, msd, dev, stream), 3)
+    floor_us, graph_us = launch_floor_us(torch, msd, dev, stream)
+    out["config"]["launch_floor_us"] = round(floor_us, 3)
+    out["config"]["graph_launch_us"] = round(graph_us, 2)
     tables = set() if args.no_shapes else set(t for t in args.tables.split(",") if t)
     if "shapes" in tables:
         out["shapes"] = shape_table(torch, msd, dev, stream)
