@@ -288,7 +288,7 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
                                         const float *__restrict__ beta, const GnScratch &scratch,
                                         const GnParams &p, uint32_t unit, uint32_t slice,
                                         uint32_t v_begin, uint32_t v_end, float *red_a,
-                                        float *red_b, float *red_c, float *stats, float *aff) {
+                                        float *red_b, float *red_c, float *stats, float2 *aff) {
     constexpr int EPV = Store<T>::EPV;
     const uint32_t tid = threadIdx.x;
     const uint32_t nt = blockDim.x;
@@ -365,8 +365,7 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
         }
     } else {
         for (uint32_t c = tid; c < p.ch_per_group; c += nt) {  // ch_per_group <= kGnLdsChannels (host)
-            aff[c] = gamma[ch0 + c];
-            aff[kGnLdsChannels + c] = beta[ch0 + c];
+            aff[c] = make_float2(gamma[ch0 + c], beta[ch0 + c]);
         }
     }
 
@@ -409,8 +408,9 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
         float g_next = 0.0f, b_next = 0.0f;
         if (!kPrefetchAffine) {
             const uint32_t c = fast_div(vidx(0, lane_again()), p.hw_vec);
-            g_next = aff[c];
-            b_next = aff[kGnLdsChannels + c];
+            const float2 gb = aff[c];  // one 8-byte LDS read
+            g_next = gb.x;
+            b_next = gb.y;
         }
 #pragma unroll
         for (int k = 0; k < K; k++) {
@@ -423,8 +423,9 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
                 b_k = b_next;
                 if (k + 1 < K) {  // the next vector's pair: its LDS latency passes under this vector's work
                     const uint32_t c = fast_div(vidx(k + 1, lane_again()), p.hw_vec);
-                    g_next = aff[c];
-                    b_next = aff[kGnLdsChannels + c];
+                    const float2 gb = aff[c];
+                    g_next = gb.x;
+                    b_next = gb.y;
                 }
             }
             const float a = rstd * g_k;
@@ -463,7 +464,7 @@ __global__ __launch_bounds__(kGnMaxThreads, (K <= (sizeof(T) == 2 ? 5 : 4) ? 8 :
     __shared__ float red_b[kGnMaxThreads / kWave];
     __shared__ float red_c[kGnMaxThreads / kWave];
     __shared__ float stats[2];
-    __shared__ float aff[K <= kGnPrefetchAffineK ? 1 : 2 * kGnLdsChannels];  // gamma, beta of the group
+    __shared__ float2 aff[K <= kGnPrefetchAffineK ? 1 : kGnLdsChannels];  // (gamma, beta) of the group's channels
     const uint32_t unit = blockIdx.x >> p.split_shift;
     const uint32_t slice = blockIdx.x & (p.split - 1);
     const uint32_t v_begin = slice * p.vec_per_slice;
