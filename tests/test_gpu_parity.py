@@ -153,8 +153,16 @@ def test_groupnorm_large_batch_plan_and_wide_groups(msd, orc, cuda):
     lib = msd.load_library()
     x = orc.normal((17, 320, 64, 64), seed=521, sigma=1.2, mean=-0.3)
     g, b = _affine(orc, 320, 521)
+    assert msd.groupnorm_plan(17, 320, 4096) == (1, 256, 20)
     _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, True)
     _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, False)
+    # the other unit sizes of the UNet at that batch: 10 and 5 vectors per lane, ragged 16 and 8
+    for channels, hw, plan in ((640, 1024, (1, 256, 10)), (1280, 256, (1, 256, 5)), (960, 1024, (1, 256, 16)),
+                               (1920, 256, (1, 256, 8))):
+        assert msd.groupnorm_plan(17, channels, hw) == plan
+        xs = orc.normal((17, channels, hw), seed=523 + channels, sigma=1.4, mean=0.2)
+        gs, bs = _affine(orc, channels, 523 + channels)
+        _run_groupnorm(msd, orc, cuda, xs, gs, bs, 32, 1e-5, True, True)
     wide = orc.normal((1, 32 * 1100, 16), seed=522, sigma=1.0)
     gw, bw = _affine(orc, 32 * 1100, 522)
     try:
