@@ -437,6 +437,7 @@ def load_nn_library(path=None):
         "msdnn_linear_init": (it, [vp]),
         "msdnn_linear_init_from": (it, [vp, flp, sz, flp, sz]),
         "msdnn_linear_forward": (it, [vp, vp, sz, vp, sz, it, it, it]),
+        "msdnn_linear_forward_grouped": (it, [ctypes.POINTER(vp), sz, vp, sz, ctypes.POINTER(vp), szp, it, it, it]),
         "msdnn_linear_destroy": (None, [vp]),
         "msdnn_softmax": (it, [vp, vp, vp, sz, it, sz, it]),
         "msdnn_ddim_sample": (it, [vp, vp, sz, it, it, MODEL_FN, vp, vp]),

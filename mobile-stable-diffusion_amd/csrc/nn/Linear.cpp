@@ -64,4 +64,47 @@ int Linear::forwardSilu(const DeviceBuffer &input, DeviceBuffer &output, bool si
     return MSD_OK;
 }
 
+int Linear::forwardSiluGrouped(const std::vector<Linear *> &layers, const DeviceBuffer &input,
+                               std::vector<DeviceBuffer> &outputs, bool silu_on_input, bool silu_on_output,
+                               unsigned num_events_in_list, const hipEvent_t *event_wait_list,
+                               hipEvent_t event) {
+    if (layers.empty()) return MSD_OK;
+    if (layers.size() != outputs.size()) throw std::runtime_error("Linear: one output per layer");
+    const Linear &first = *layers[0];
+    const size_t K = first.weightShape[1];
+    if (K == 0 || input.count() % K != 0) throw std::runtime_error("inputSize % weightShape[1] != 0");
+    const size_t M = input.count() / K;
+    if (M > 8) throw std::runtime_error("Linear: more than 8 input rows is a GEMM, which this library leaves out");
+    std::vector<const void *> ws(layers.size());
+    std::vector<const float *> bs(layers.size());
+    std::vector<void *> ys(layers.size());
+    std::vector<size_t> ns(layers.size());
+    for (size_t i = 0; i < layers.size(); i++) {
+        const Linear &l = *layers[i];
+        if (l.bufferWeight.empty()) throw std::runtime_error("Linear: init() not called");
+        if (l.weightShape[1] != K || l.dtype != first.dtype || l.stream != first.stream)
+            throw std::runtime_error("Linear: grouped layers differ in in_features, storage type or stream");
+        if (input.dtype() != l.dtype || outputs[i].dtype() != l.dtype)
+            throw std::runtime_error("Linear: buffer storage type != weight storage type");
+        if (input.ptr() == outputs[i].ptr()) throw std::runtime_error("Linear not support input == output");
+        if (outputs[i].count() != M * l.weightShape[0])
+            throw std::runtime_error("Linear: output size != M * weightShape[0]");
+        ws[i] = l.bufferWeight.ptr();
+        bs[i] = l.bufferBias.empty() ? nullptr : static_cast<const float *>(l.bufferBias.ptr());
+        ys[i] = outputs[i].ptr();
+        ns[i] = l.weightShape[0];
+    }
+    for (unsigned i = 0; i < num_events_in_list; i++) {
+        const hipError_t err = hipStreamWaitEvent(first.stream, event_wait_list[i], 0);
+        if (err != hipSuccess) return (int)err;
+    }
+    const int rc = msd_linear_rows_grouped(input.ptr(), ws.data(), bs.data(), ys.data(), ns.data(), layers.size(), M,
+                                           K, silu_on_input ? MSD_ACT_SILU : MSD_ACT_NONE,
+                                           silu_on_output ? MSD_ACT_SILU : MSD_ACT_NONE, (int)first.dtype,
+                                           first.stream);
+    if (rc != MSD_OK) return rc;
+    if (event) return (int)hipEventRecord(event, first.stream);
+    return MSD_OK;
+}
+
 }  // namespace msd

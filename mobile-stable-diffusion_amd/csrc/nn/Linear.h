@@ -40,6 +40,16 @@ public:
                     bool silu_on_output, unsigned num_events_in_list = 0,
                     const hipEvent_t *event_wait_list = nullptr, hipEvent_t event = nullptr);
 
+    // Several layers on the SAME input rows in one launch: outputs[i] = layers[i](input), each
+    // exactly what its own forwardSilu() call gives.  For the embed_linear of all ResBlocks of a
+    // UNet step, which the reference runs one by one on the same emb (M/nn/ResBlock.cpp:173-183;
+    // emb exists once M/UNetModel.cpp:1107-1120 has run): call it once ahead of the blocks.
+    // All layers share in_features, the storage type and the stream; throws what forwardSilu throws.
+    static int forwardSiluGrouped(const std::vector<Linear *> &layers, const DeviceBuffer &input,
+                                  std::vector<DeviceBuffer> &outputs, bool silu_on_input, bool silu_on_output,
+                                  unsigned num_events_in_list = 0, const hipEvent_t *event_wait_list = nullptr,
+                                  hipEvent_t event = nullptr);
+
     std::vector<size_t> weightShape;  // {out_features, in_features}
 
 private:

@@ -234,6 +234,20 @@ int msdnn_linear_forward(void *h, void *in, size_t in_bytes, void *out, size_t o
         return static_cast<Linear *>(h)->forwardSilu(i, o, silu_on_input != 0, silu_on_output != 0);
     });
 }
+// `count` Linear handles on the same input rows in one launch; outs / out_bytes are host arrays
+int msdnn_linear_forward_grouped(void *const *hs, size_t count, void *in, size_t in_bytes, void *const *outs,
+                                 const size_t *out_bytes, int dtype, int silu_on_input, int silu_on_output) {
+    return guarded([&] {
+        std::vector<Linear *> layers(count);
+        std::vector<DeviceBuffer> outputs;
+        for (size_t i = 0; i < count; i++) {
+            layers[i] = static_cast<Linear *>(hs[i]);
+            outputs.push_back(wrap(outs[i], out_bytes[i], dtype));
+        }
+        const DeviceBuffer input = wrap(in, in_bytes, dtype);
+        return Linear::forwardSiluGrouped(layers, input, outputs, silu_on_input != 0, silu_on_output != 0);
+    });
+}
 void msdnn_linear_destroy(void *h) { delete static_cast<Linear *>(h); }
 
 // ---- row softmax

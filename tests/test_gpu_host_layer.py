@@ -197,6 +197,47 @@ def test_step_runner_eager_and_graph(msd, nn, cuda):
 
 # ----------------------------------------------------------------- neighbours of the path
 @pytest.mark.parametrize("half", [False, True], ids=["f32", "f16"])
+def test_linear_objects_grouped_forward_equals_one_call_per_layer(msd, nn, orc, cuda, half):
+    """Linear::forwardSiluGrouped: the embed_linear of several ResBlocks on the same emb in one
+    launch (M/nn/ResBlock.cpp:173-183), bit for bit what each layer's own forwardSilu gives."""
+    import ctypes
+    import torch
+    couts = [320, 640, 1280, 1280, 640]
+    fp = ctypes.POINTER(ctypes.c_float)
+    dt = torch.float16 if half else torch.float32
+    es = 2 if half else 4
+    layers = []
+    for i, n in enumerate(couts):
+        l = nn.msdnn_linear_create(None, 1280, n, None, None, int(half))
+        w = orc.normal((n, 1280), seed=700 + i, sigma=1280 ** -0.5)
+        b = orc.normal((n,), seed=720 + i, sigma=0.1)
+        assert l and nn.msdnn_linear_init_from(l, w.ctypes.data_as(fp), w.size, b.ctypes.data_as(fp), b.size) == 0
+        layers.append(l)
+    emb = torch.randn((2, 1280), device=cuda, generator=torch.Generator(device=cuda).manual_seed(5)).to(dt)
+    single = [torch.empty((2, n), dtype=dt, device=cuda) for n in couts]
+    grouped = [torch.empty((2, n), dtype=dt, device=cuda) for n in couts]
+    try:
+        for l, o in zip(layers, single):
+            assert nn.msdnn_linear_forward(l, _ptr(emb), emb.numel() * es, _ptr(o), o.numel() * es, int(half), 1, 0) == 0
+        hs = (ctypes.c_void_p * len(layers))(*layers)
+        outs = (ctypes.c_void_p * len(layers))(*[o.data_ptr() for o in grouped])
+        nbytes = (ctypes.c_size_t * len(layers))(*[o.numel() * es for o in grouped])
+        assert nn.msdnn_linear_forward_grouped(hs, len(layers), _ptr(emb), emb.numel() * es, outs, nbytes, int(half),
+                                               1, 0) == 0, msd.nn_last_error()
+        torch.cuda.synchronize()
+        for a, b in zip(single, grouped):
+            assert torch.equal(a, b)
+        # refusals: one output per layer with the layer's size; the input is not an output
+        nbytes[1] = 16
+        assert nn.msdnn_linear_forward_grouped(hs, len(layers), _ptr(emb), emb.numel() * es, outs, nbytes, int(half),
+                                               1, 0) < 0
+        assert "output size" in msd.nn_last_error()
+    finally:
+        for l in layers:
+            nn.msdnn_linear_destroy(l)
+
+
+@pytest.mark.parametrize("half", [False, True], ids=["f32", "f16"])
 def test_linear_objects_run_the_time_embedding_mlp(msd, nn, orc, cuda, tmp_path, half):
     """time_embed_0 + SiLU, time_embed_2, then a ResBlock's SiLU + embed_linear, weights from .npy."""
     import torch
