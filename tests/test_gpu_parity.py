@@ -173,6 +173,47 @@ def test_groupnorm_large_batch_plan_and_wide_groups(msd, orc, cuda):
     assert msd.status() == 0
 
 
+@pytest.mark.parametrize("half", [False, True], ids=["f32", "f16"])
+def test_groupnorm_and_layernorm_non_finite_inputs_poison_their_unit_only(msd, orc, cuda, half):
+    """An infinity or a NaN in the input makes the statistics of its (sample, group) / row NaN in
+    the reference's arithmetic (K/group_norm.cl:1-76, K/layer_norm.cl:1-78: inf - inf), so that unit
+    comes out all NaN and every other unit is untouched; the same must hold here, for whole units
+    and for units cut in slices (the slices exchange the NaN)."""
+    x = orc.normal((2, 320, 64, 64), seed=641, sigma=1.0)
+    x[0, 5, 3, 7] = np.inf          # group 0 of sample 0
+    x[1, 315, 60, 1] = np.nan       # group 31 of sample 1
+    x[1, 100, 0, 0] = -np.inf       # group 10 of sample 1
+    g, b = _affine(orc, 320, 641)
+    xin = orc.round_to_half(x) if half else x
+    for shape in ((2, 320, 64, 64), (2, 320, 16, 16)):
+        xs = np.ascontiguousarray(xin[:, :, :shape[2], :shape[3]])
+        ref = orc.groupnorm(xs, g, b, 32, 1e-5, True)
+        got = msd.groupnorm(_to_dev(xs, cuda, half), _to_dev(g, cuda), _to_dev(b, cuda), 32, 1e-5, True).float().cpu().numpy()
+        assert np.array_equal(np.isnan(got), np.isnan(ref))
+        bad = np.isnan(ref).reshape(2, 32, -1)
+        poisoned = (~np.isfinite(xs)).reshape(2, 32, -1).any(axis=2)
+        assert poisoned.sum() >= 2
+        assert np.array_equal(bad.all(axis=2), poisoned) and np.array_equal(bad.any(axis=2), poisoned)
+        ok = ~np.isnan(ref)
+        if half:
+            assert_close_f16(got[ok], ref[ok], "groupnorm f16 with non-finite units")
+        else:
+            assert_close_f32(got[ok], ref[ok], what="groupnorm f32 with non-finite units")
+    rows = xin.reshape(-1, 320)[:4096].copy()
+    rows[7, 300] = np.inf
+    rows[4000, 0] = np.nan
+    ref = orc.layernorm(rows, g, b, 1e-5)
+    got = msd.layernorm(_to_dev(rows, cuda, half), _to_dev(g, cuda), _to_dev(b, cuda), 1e-5).float().cpu().numpy()
+    assert np.array_equal(np.isnan(got), np.isnan(ref))
+    ok = ~np.isnan(ref)
+    assert np.isnan(ref).all(axis=1).sum() >= 2
+    if half:
+        assert_close_f16(got[ok], ref[ok], "layernorm f16 with non-finite rows")
+    else:
+        assert_close_f32(got[ok], ref[ok], what="layernorm f32 with non-finite rows")
+    assert msd.status() == 0
+
+
 @pytest.mark.parametrize("split", [2, 4, 16])
 def test_groupnorm_slice_that_stops_waiting_computes_its_siblings_statistics(msd, orc, cuda, split):
     """With a poll limit of one, nearly every workgroup gives up on its siblings at once and
