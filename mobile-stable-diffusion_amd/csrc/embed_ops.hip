@@ -287,18 +287,19 @@ __global__ __launch_bounds__(kSmThreads) void softmax_short_kernel(const T *x, T
 // Short rows whose length is not a multiple of a 16-byte vector (77 text tokens): a
 // workgroup takes RB consecutive rows (RB a multiple of 8) as one flat, 16-byte aligned
 // run of memory (such a block is a whole number of vectors for any row length), moves it
-// through LDS with full vectors, and a team of 4 lanes per row does the arithmetic on
-// the LDS copy.
-constexpr int kSmFlatTeam = 4;
-constexpr uint32_t kSmFlatMaxCols = 128;  // RB = 64: 32 KiB of LDS
+// through LDS with full vectors, and a team of 4, 8 or 16 lanes per row does the arithmetic
+// on the LDS copy.
+constexpr uint32_t kSmFlatMaxCols = 128;  // RB = 64: 16 or 32 KiB of LDS
 
-template <typename T, int RB, int ITERS>
-__global__ __launch_bounds__(RB * kSmFlatTeam) void softmax_flat_kernel(const T *x, T *y, uint32_t cols,
-                                                                       int stable) {
+template <typename T, int RB, int ITERS, int TEAM>
+__global__ __launch_bounds__(RB * TEAM) void softmax_flat_kernel(const T *x, T *y, uint32_t cols, int stable) {
     constexpr int EPV = Store<T>::EPV;
-    constexpr int NT = RB * kSmFlatTeam;
+    constexpr int NT = RB * TEAM;
     constexpr int UN = 4;
-    extern __shared__ float tile[];  // [RB][cols], cols <= ITERS * kSmFlatTeam
+    // [RB][cols] in the storage type: whole vectors go in and out as they are (one 16-byte LDS
+    // access per vector), only the arithmetic in between touches single elements
+    extern __shared__ u32x4 tile_vec[];
+    T *tile = reinterpret_cast<T *>(tile_vec);
     const uint32_t block_vecs = RB * cols / EPV;
     const size_t first = (size_t)blockIdx.x * block_vecs;
     const u32x4 *in = reinterpret_cast<const u32x4 *>(x) + first;
@@ -310,29 +311,24 @@ __global__ __launch_bounds__(RB * kSmFlatTeam) void softmax_flat_kernel(const T 
 #pragma unroll
         for (int u = 0; u < UN; u++) {
             const uint32_t v = base + u * NT;
-            if (v < block_vecs) {
-                float f[EPV];
-                Store<T>::unpack(raw[u], f);
-#pragma unroll
-                for (int e = 0; e < EPV; e++) tile[v * EPV + e] = f[e];
-            }
+            if (v < block_vecs) tile_vec[v] = raw[u];
         }
     }
     __syncthreads();
     // the lane's share of its row, from LDS into registers with independent reads
-    float *row = tile + (threadIdx.x / kSmFlatTeam) * cols;
-    const uint32_t j = threadIdx.x % kSmFlatTeam;
+    T *row = tile + (threadIdx.x / TEAM) * cols;
+    const uint32_t j = threadIdx.x % TEAM;
     float f[ITERS];
     float mx = kNegInf;
 #pragma unroll
     for (int i = 0; i < ITERS; i++) {
-        const uint32_t c = j + i * kSmFlatTeam;
-        f[i] = c < cols ? row[c] : kNegInf;
+        const uint32_t c = j + i * TEAM;
+        f[i] = c < cols ? Store<T>::load1(row + c) : kNegInf;
         mx = fmaxf(mx, f[i]);
     }
     float shift = 0.0f;
     if (stable) {
-        mx = team_max<kSmFlatTeam>(mx);
+        mx = team_max<TEAM>(mx);
         shift = mx == kNegInf ? 0.0f : mx;
     }
     const float bias = -shift * kLog2e;
@@ -342,32 +338,25 @@ __global__ __launch_bounds__(RB * kSmFlatTeam) void softmax_flat_kernel(const T 
         f[i] = __builtin_amdgcn_exp2f(fmaf(f[i], kLog2e, bias));
         total += f[i];
     }
-    total = team_sum<kSmFlatTeam>(total);
+    total = team_sum<TEAM>(total);
     const float inv = 1.0f / total;
 #pragma unroll
     for (int i = 0; i < ITERS; i++) {
-        const uint32_t c = j + i * kSmFlatTeam;
-        if (c < cols) row[c] = f[i] * inv;
+        const uint32_t c = j + i * TEAM;
+        if (c < cols) Store<T>::store1(row + c, f[i] * inv);
     }
     __syncthreads();
-    for (uint32_t v = threadIdx.x; v < block_vecs; v += NT) {
-        float g[EPV];
-#pragma unroll
-        for (int e = 0; e < EPV; e++) g[e] = tile[v * EPV + e];
-        store_stream(out + v, Store<T>::pack(g));
-    }
+    for (uint32_t v = threadIdx.x; v < block_vecs; v += NT) store_stream(out + v, tile_vec[v]);
 }
 
-template <typename T, int ITERS>
-void softmax_flat_launch(const T *x, T *y, uint32_t blocks, uint32_t rb, uint32_t cols, int stable,
-                         hipStream_t stream) {
-    const size_t lds = (size_t)rb * cols * sizeof(float);
-    if (rb == 64)
-        hipLaunchKernelGGL((softmax_flat_kernel<T, 64, ITERS>), dim3(blocks), dim3(256), lds, stream, x, y, cols, stable);
-    else if (rb == 32)
-        hipLaunchKernelGGL((softmax_flat_kernel<T, 32, ITERS>), dim3(blocks), dim3(128), lds, stream, x, y, cols, stable);
+template <typename T, int RB, int TEAM>
+void softmax_flat_launch(const T *x, T *y, uint32_t blocks, uint32_t cols, int stable, hipStream_t stream) {
+    const size_t lds = (size_t)RB * cols * sizeof(T);  // a whole number of 16-byte vectors: RB is a multiple of 8
+    constexpr int kFew = (80 + TEAM - 1) / TEAM, kMany = kSmFlatMaxCols / TEAM;
+    if (cols <= 80)
+        hipLaunchKernelGGL((softmax_flat_kernel<T, RB, kFew, TEAM>), dim3(blocks), dim3(RB * TEAM), lds, stream, x, y, cols, stable);
     else
-        hipLaunchKernelGGL((softmax_flat_kernel<T, 16, ITERS>), dim3(blocks), dim3(64), lds, stream, x, y, cols, stable);
+        hipLaunchKernelGGL((softmax_flat_kernel<T, RB, kMany, TEAM>), dim3(blocks), dim3(RB * TEAM), lds, stream, x, y, cols, stable);
 }
 
 // ---------------------------------------------------------------------------
@@ -556,17 +545,33 @@ int softmax_dispatch(const void *xv, void *yv, size_t rows, size_t cols, int sta
         else softmax_team_launch<T, 16, 64>(x, y, r, rv, stable, stream);
         return launch_status();
     }
-    // The flat kernel pays two LDS round trips per row; it wins once the launch is large
-    // enough for the row-per-wavefront kernel to be bound by its 2-byte accesses
-    // (measured crossover near 20000 rows of 77).  A set knob forces it for any size.
+    // The flat kernel pays two barriers and two LDS round trips; below about 12000 rows the
+    // row-per-wavefront kernel is quicker (3.08 against 3.10 us at 10240 x 77, 3.26 against 3.18
+    // at 12288).  Lanes per row: as many as keep the launch within the 8192 wavefronts the chip
+    // holds at once (a second round of wavefronts costs more than the shorter serial chain per
+    // lane gains: 16 lanes per row take 4.09 us at 32768 x 77 and 7.08 at 65536, 8 lanes 4.52 and
+    // 5.76); past one round 4 lanes per row are the cheapest for up to 80 columns, 8 beyond.
+    // A set knob forces the flat kernel and its rows per workgroup for any size.
     const int tune_rows = g_tuning.softmax_rows.load(std::memory_order_relaxed);
-    const uint32_t rb = tune_rows ? (uint32_t)tune_rows : 64u;
-    const bool flat_pays = tune_rows ? rows >= rb : rows >= 24576;
+    const uint32_t team = rows <= 32768 ? 16u : rows <= 65536 ? 8u : cols <= 80 ? 4u : 8u;
+    // workgroups of 512 lanes up to 80 columns, of 256 beyond, and at most 64 rows
+    const uint32_t lanes = cols <= 80 ? 512u : 256u;
+    const uint32_t rb = tune_rows ? (uint32_t)tune_rows : lanes / team > 64u ? 64u : lanes / team;
+    const bool flat_pays = tune_rows ? rows >= rb : rows >= 12288;
     if (cols <= kSmFlatMaxCols && cols >= 8 && flat_pays && aligned16(x) && aligned16(y)) {
         // whole blocks of rb rows through the flat kernel, the rest (if any) row by row below
         const uint32_t blocks = r / rb;
-        if (c <= 20 * kSmFlatTeam) softmax_flat_launch<T, 20>(x, y, blocks, rb, c, stable, stream);
-        else softmax_flat_launch<T, 32>(x, y, blocks, rb, c, stable, stream);
+        switch (team * 100 + rb) {
+            case 464: softmax_flat_launch<T, 64, 4>(x, y, blocks, c, stable, stream); break;
+            case 432: softmax_flat_launch<T, 32, 4>(x, y, blocks, c, stable, stream); break;
+            case 416: softmax_flat_launch<T, 16, 4>(x, y, blocks, c, stable, stream); break;
+            case 864: softmax_flat_launch<T, 64, 8>(x, y, blocks, c, stable, stream); break;
+            case 832: softmax_flat_launch<T, 32, 8>(x, y, blocks, c, stable, stream); break;
+            case 816: softmax_flat_launch<T, 16, 8>(x, y, blocks, c, stable, stream); break;
+            case 1664: softmax_flat_launch<T, 64, 16>(x, y, blocks, c, stable, stream); break;
+            case 1632: softmax_flat_launch<T, 32, 16>(x, y, blocks, c, stable, stream); break;
+            default: softmax_flat_launch<T, 16, 16>(x, y, blocks, c, stable, stream); break;
+        }
         const uint32_t done = blocks * rb;
         if (done == r) return launch_status();
         x += (size_t)done * c;

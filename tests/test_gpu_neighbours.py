@@ -243,6 +243,22 @@ def test_softmax_short_rows_flat_kernel(msd, orc, cuda, rb):
     assert lib.msd_set_tuning(msd.TUNE_SOFTMAX_ROWS, 48) == 1
 
 
+@pytest.mark.parametrize("rows,cols,half,knob", [
+    (12288 + 7, 77, True, 0), (20000, 100, False, 0),    # 16 lanes per row, 32 / 16 rows per workgroup
+    (40000 + 3, 77, False, 0), (40000, 100, True, 0),    # 8 lanes per row, 64 / 32 rows
+    (66000 + 1, 77, True, 0), (66000, 100, True, 0),     # 4 lanes per row up to 80 columns, 8 beyond
+    (66000, 77, False, 16), (66000, 33, True, 32), (40000, 127, True, 16), (40000, 9, False, 64)])
+def test_softmax_flat_kernel_lanes_per_row(msd, orc, cuda, rows, cols, half, knob):
+    """Row counts on both sides of the limits where the flat kernel changes its lanes per row."""
+    lib = msd.load_library()
+    assert lib.msd_set_tuning(msd.TUNE_SOFTMAX_ROWS, knob) == 0
+    try:
+        for stable in (0, 1):
+            _softmax_case(msd, orc, cuda, rows, cols, 8500 + cols + stable, half, stable, inplace=bool(stable))
+    finally:
+        assert lib.msd_set_tuning(msd.TUNE_SOFTMAX_ROWS, 0) == 0
+
+
 def test_softmax_cross_attention_full_rows(msd, orc, cuda):
     """All 2 x 8 x 4096 query rows against 77 text tokens (the size that takes the flat kernel)."""
     _softmax_case(msd, orc, cuda, 2 * 8 * 4096, 77, 8400, True, 0, inplace=True)
