@@ -693,13 +693,17 @@ int k_for(uint32_t vecs, uint32_t threads, uint32_t max_k, bool equal_slices) {
     return k;
 }
 
-// 640 ... 1024 lanes that hold a slice of `vecs` vectors as exactly one or two vectors per lane
-// (nothing masked), 0 if there is no such size.  Measured against the next power-of-two size
-// with a masked tail: 1280-vector slices 5.97 us on 640 lanes against 6.20 on 1024, 1920-vector
-// units 4.24 us on 960 lanes against 4.35 on 512.
-uint32_t exact_fit_threads(uint32_t vecs) {
-    for (uint32_t t = kGnMaxThreads; t >= 640; t -= kWave)
-        if (vecs == t || vecs == 2 * t) return t;
+// 640 ... 1024 lanes that hold a slice of `vecs` vectors as exactly 1 ... max_fit_k vectors per
+// lane (nothing masked), 0 if there is no such size.  Measured against the next power-of-two
+// size with a masked tail, 2-byte elements: 1280-vector slices 5.97 us on 640 lanes against 6.20
+// on 1024, 1920-vector units 4.24 us on 960 lanes against 4.35 on 512 (three or four vectors per
+// lane gain nothing there).  4-byte elements gain up to four vectors per lane: 3840-vector slices
+// 12.28 us on 960 x 4 against 12.55 on 512 x 8, 2560-vector slices 7.12 on 640 x 4 against 7.23
+// on 1024 x 3.
+uint32_t exact_fit_threads(uint32_t vecs, uint32_t max_fit_k) {
+    for (uint32_t k = 1; k <= max_fit_k; k++)
+        for (uint32_t t = kGnMaxThreads; t >= 640; t -= kWave)
+            if (vecs == k * t) return t;
     return 0;
 }
 
@@ -709,7 +713,7 @@ uint32_t exact_fit_threads(uint32_t vecs) {
 // larger slices want 1024 lanes, and a small whole unit runs best with exactly one vector per
 // lane.  The tail of a slice that does not fill K * threads is masked.
 GnPlan plan_slice(uint32_t vecs, uint32_t split, uint32_t force_threads, uint32_t max_k, bool equal_slices,
-                  size_t blocks = 0) {
+                  size_t blocks = 0, size_t elt = 2) {
     GnPlan pl{split, 0, 0};
     if (force_threads && k_for(vecs, force_threads, max_k, equal_slices) != 0) {
         pl.threads = force_threads;
@@ -722,15 +726,23 @@ GnPlan plan_slice(uint32_t vecs, uint32_t split, uint32_t force_threads, uint32_
         // 18.4, 1920: 12.0 / 13.1 / 15.4, 3840: 23.3 / 24.9 / 24.9; fp32 5120: 29.5 / 29.8 / 33.9.
         // Batch 16 (512 units), 5120: 14.95 / 15.2 / 15.2; batch 12 is where 256 lanes lose
         // (13.9 / 13.3 / 13.4) and the rules below take over.
+        // Exactly two or three workgroups per CU that are slices of cut units (4-byte elements at
+        // batch 2 - 8) still want large workgroups: 3840-vector slices 12.28 us on 960 x 4 against
+        // 12.55 on 512 x 8, 5120-vector slices 14.6 us on 512 x 10 against 14.8 on 640 x 8.
+        const bool cut_few = split > 1 && blocks < 4 * kChipCus;
+        if (cut_few) pl.threads = exact_fit_threads(vecs, elt == 2 ? 2 : 4);
         for (uint32_t t : {256u, 512u, 768u, 1024u}) {
-            if (k_for(vecs, t, max_k, equal_slices) == 0) continue;
+            if (pl.threads != 0) break;
+            if ((cut_few && t == 256u) || k_for(vecs, t, max_k, equal_slices) == 0) continue;
             pl.threads = t;
-            break;
         }
         if (pl.threads == 0) pl.threads = kGnMaxThreads;
-    } else if (uint32_t exact = (split == 1 && vecs == 1280) ? 0u : exact_fit_threads(vecs)) {
-        // (a whole unit of 1280 vectors is the exception: 3.55 us on 512 lanes with a masked tail
-        // against 3.62 us on 640 x 2)
+    } else if (uint32_t exact = (split == 1 && vecs == (elt == 2 ? 1280u : 2560u))
+                                    ? 0u
+                                    : exact_fit_threads(vecs, elt == 2 ? 2 : 4)) {
+        // (a whole unit of 10240 elements is the exception.  2-byte elements: 3.55 us on 512
+        // lanes with a masked tail against 3.62 us on 640 x 2; 4-byte elements: 512 x 5 is an
+        // exact fit itself, 3.98 us against 4.08 on 640 x 4)
         pl.threads = exact;
     } else if (vecs > 512u * 5u || (split > 1 && vecs >= 960))  // slices of a cut unit: 2 - 3 % faster
         pl.threads = kGnMaxThreads;
@@ -805,11 +817,32 @@ GnDecision gn_decide(size_t elt, size_t batch, size_t channels, size_t hw, size_
         // With 256 or more units every CU has one of its own and cutting only adds the exchange
         // (batch 8, 320 channels at 64x64: 9.0 us whole against 10.5 us in two).
         uint32_t want = 1;
-        if (unit_size > 24576) {
-            // (up to 32 Ki elements two slices are enough: 960 channels at 32 x 32, 5.40 us in two
-            // against 5.63 us in four)
-            want = units >= 256 ? 1 : (units >= 128 || unit_size <= 32768) ? 2 : 4;
-            if (units * 4 < 192 && unit_size >= 65536) want = 8;
+        if (elt == 2) {
+            if (unit_size > 24576) {
+                // (up to 32 Ki elements two slices are enough from 64 units on: 960 channels at
+                // 32 x 32, batch 2, 5.40 us in two against 5.63 us in four; batch 1 4.86 in four
+                // against 5.03 in two)
+                want = units >= 256 ? 1 : (units >= 128 || (unit_size <= 32768 && units >= 64)) ? 2 : 4;
+                // (batch 1: 960 channels at 64 x 64 7.08 us in eight against 7.16 in four, 640
+                // channels 6.56 against 6.12)
+                if (units * 4 < 192 && unit_size > 98304) want = 8;
+            }
+        } else {
+            // 4-byte elements, half the arithmetic per vector: whole up to 5120 vectors (4096 when
+            // the units alone fill less than a quarter of the chip), then halved until the slices
+            // are at most 5120 vectors or the launch would pass two workgroups per CU; a launch
+            // of fewer than 128 workgroups goes on halving down to 960-vector slices.  Measured
+            // per launch, batch 1 / 2 / 4: 960 channels at 64 x 64 (30720 vectors) 8.8 us in
+            // eight against 8.8 in four / 12.3 in eight against 13.4 in four / 21.3 in four
+            // against 23.9 in two; 640 channels at 32 x 32 (5120) 5.12 in four against 5.40 whole /
+            // 5.69 whole against 5.81 in two / 6.10 whole.
+            const size_t whole_limit = units < 64 ? 4096 : 5120;
+            for (;;) {
+                const size_t slice = (vec_per_unit + want - 1) / want;
+                const size_t limit = want == 1 ? whole_limit : units * want < 128 ? 1919 : 5120;
+                if (units * want * 2 > 2 * kChipCus || slice <= limit || slice / 2 < 960 || want >= kGnMaxSplit) break;
+                want *= 2;
+            }
         }
         // Large batches of very long units (more than 10240 vectors): slices of up to 5120
         // vectors on 256 lanes overlap better than whole units on 768 - 1024 lanes, the exchange
@@ -830,7 +863,7 @@ GnDecision gn_decide(size_t elt, size_t batch, size_t channels, size_t hw, size_
         (size_t)tune_threads * kMaxK >= vec_per_slice)
         force_threads = (uint32_t)tune_threads;
     const bool equal_slices = vec_per_slice * split == vec_per_unit;
-    const GnPlan pl = plan_slice((uint32_t)vec_per_slice, split, force_threads, kMaxK, equal_slices, units * split);
+    const GnPlan pl = plan_slice((uint32_t)vec_per_slice, split, force_threads, kMaxK, equal_slices, units * split, elt);
     if (pl.k == 0 || (pl.k > kGnPrefetchAffineK && cpg > kGnLdsChannels)) return d;
     d.split = split;
     d.threads = pl.threads;

@@ -632,6 +632,20 @@ def test_groupnorm_larger_batches_pick_other_splits(msd, orc, cuda, batch, chann
     assert msd.status() == 0
 
 
+@pytest.mark.parametrize("batch,channels,hw,plan", [
+    (1, 320, 4096, (4, 640, 4)), (1, 640, 1024, (4, 640, 2)), (1, 960, 4096, (8, 960, 4)),
+    (2, 960, 4096, (8, 960, 4)), (2, 320, 4096, (2, 1024, 5)), (2, 1920, 256, (1, 960, 4)),
+    (2, 640, 256, (1, 640, 2)), (4, 640, 4096, (4, 512, 10)), (4, 1920, 1024, (4, 960, 4)),
+    (8, 320, 4096, (2, 512, 10)), (8, 640, 4096, (2, 512, 20))])
+def test_groupnorm_fp32_plans_at_unet_shapes(msd, orc, cuda, batch, channels, hw, plan):
+    """4-byte elements are cut more often and into exact fits of up to four vectors per lane."""
+    assert msd.groupnorm_plan(batch, channels, hw, 32, msd.DTYPE_F32) == plan
+    x = orc.normal((batch, channels, hw), seed=batch * 1000 + channels + hw, sigma=2.0, mean=-0.1)
+    g, b = _affine(orc, channels, 78)
+    _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half=False)
+    assert msd.status() == 0
+
+
 def test_groupnorm_many_units_and_register_limits(msd, orc, cuda):
     # more units than scratch slots (never split), and float units that need a split to fit
     for shape, groups, half in [((300, 64, 4, 8), 32, True),     # 9600 units

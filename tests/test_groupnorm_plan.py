@@ -47,7 +47,9 @@ def test_plans_of_the_unet_shapes_at_batch_2_and_32():
     expected = {
         (2, 320, 4096, f16): (4, 640, 2), (2, 640, 1024, f16): (1, 512, 5), (2, 1280, 256, f16): (1, 512, 3),
         (2, 1280, 64, f16): (1, 320, 1), (2, 960, 1024, f16): (2, 960, 2), (2, 1920, 256, f16): (1, 960, 2),
-        (1, 320, 4096, f32): (4, 1024, 3),
+        (1, 320, 4096, f32): (4, 640, 4), (1, 640, 4096, f16): (4, 1024, 3), (1, 960, 4096, f16): (8, 960, 2),
+        (2, 960, 4096, f32): (8, 960, 4), (2, 640, 1024, f32): (1, 1024, 5), (1, 640, 1024, f32): (4, 640, 2),
+        (4, 640, 4096, f32): (4, 512, 10), (8, 640, 4096, f32): (2, 512, 20), (2, 640, 256, f32): (1, 640, 2),
         (32, 320, 4096, f16): (1, 256, 20), (32, 640, 1024, f16): (1, 256, 10), (32, 1280, 256, f16): (1, 256, 5),
         (8, 320, 4096, f16): (1, 1024, 5), (32, 960, 4096, f16): (4, 256, 16),
     }
