@@ -267,9 +267,15 @@ def _rotating_launch_us(torch, msd, stream, launch, xs, ys, warm=20, budget=2000
 
 
 def _gn_plan_text(msd, batch, channels, hw, elt):
-    """'slices per unit x lanes x vectors per lane' of the GroupNorm launch for this shape."""
-    split, threads, k = msd.groupnorm_plan(batch, channels, hw, 32, msd.DTYPE_F16 if elt == 2 else msd.DTYPE_F32)
-    return "general kernel" if split == 0 else "%d x %d lanes x %d vectors" % (split, threads, k)
+    """'slices per unit x lanes x vectors per lane' of the GroupNorm launch for this shape (output
+    apart from the input, as the tables run it), ', w writers' when w workgroups share each whole
+    unit and store a w-th of it each."""
+    split, threads, k, writers = msd.groupnorm_plan(batch, channels, hw, 32,
+                                                    msd.DTYPE_F16 if elt == 2 else msd.DTYPE_F32)
+    if split == 0:
+        return "general kernel"
+    text = "%d x %d lanes x %d vectors" % (split, threads, k)
+    return text + (", %d writers" % writers if writers > 1 else "")
 
 
 def _kernel_case(torch, msd, dev, kind, p, dt, batch):

@@ -90,6 +90,8 @@ int msd_gn_fallbacks(void *stream, unsigned int *count, int reset);
 #define MSD_TUNE_SOFTMAX_ROWS 6   /* rows per workgroup of the short-row softmax: 16, 32 or 64 */
 #define MSD_TUNE_GN_SPIN_LIMIT 7  /* polls a GroupNorm workgroup waits for a sibling before it computes
                                      that sibling's statistics itself (tests set 1 to exercise that path) */
+#define MSD_TUNE_GN_WRITERS 8     /* workgroups that share one whole (sample, group), each storing a part
+                                     of it: 1 (never), 2, 4, 8 or 16 (wherever the launch allows it) */
 int msd_set_tuning(int knob, int value);
 
 /*
@@ -123,13 +125,16 @@ int msd_groupnorm_noalloc(const void *x, void *y, const float *gamma, const floa
 /*
  * The launch msd_groupnorm (noalloc != 0: msd_groupnorm_noalloc) makes for this shape on 16-byte
  * aligned tensors, under the tuning knobs as they are set: *split workgroups per (sample, group),
- * *threads lanes each, *vectors_per_lane 16-byte vectors held per lane.  *split = 0 (the others
- * too) means the general kernel: one 256-lane workgroup per (sample, group), nothing held in
- * registers.  Host arithmetic only: needs no GPU and launches nothing.  For diagnostics, tests and
- * benchmark tables.  No counterpart in the reference (its geometry is fixed, M/nn/GroupNorm.cpp:105-128).
+ * *threads lanes each, *vectors_per_lane 16-byte vectors held per lane.  *writers > 1 (then
+ * *split = 1): that many workgroups per (sample, group) each load and reduce all of it and store
+ * one part; such a launch is only made when y does not overlap x, so in_place != 0 asks for the
+ * plan of a call with y == x.  *split = 0 (the others too) means the general kernel: one 256-lane
+ * workgroup per (sample, group), nothing held in registers.  Host arithmetic only: needs no GPU
+ * and launches nothing.  For diagnostics, tests and benchmark tables.  No counterpart in the
+ * reference (its geometry is fixed, M/nn/GroupNorm.cpp:105-128).
  */
 int msd_groupnorm_plan(size_t batch, size_t channels, size_t hw, size_t groups, int dtype, int noalloc,
-                       int *split, int *threads, int *vectors_per_lane);
+                       int in_place, int *split, int *threads, int *vectors_per_lane, int *writers);
 
 /*
  * GroupNorm whose result is stored token-major: x is [batch, channels, hw], y is

@@ -18,7 +18,7 @@ LIB_NN_PATH = os.path.join(CSRC_DIR, "libmsd_nn.so")
 DTYPE_F32 = 0
 DTYPE_F16 = 1
 TUNE_GN_SPLIT, TUNE_GN_THREADS, TUNE_LN_CHUNK, TUNE_LN_THREADS, TUNE_GEGLU_VECTORS, TUNE_ACT_VECTORS, \
-    TUNE_SOFTMAX_ROWS, TUNE_GN_SPIN_LIMIT = range(8)
+    TUNE_SOFTMAX_ROWS, TUNE_GN_SPIN_LIMIT, TUNE_GN_WRITERS = range(9)
 ERR_SCRATCH_LIMIT = -2
 
 # every symbol include/msd_hip.h declares
@@ -62,7 +62,7 @@ def load_library(path=None):
     lib.msd_set_tuning.argtypes = [it, it]
     lib.msd_groupnorm.argtypes = [vp, vp, vp, vp, sz, sz, sz, sz, fl, it, it, vp]
     lib.msd_groupnorm_noalloc.argtypes = [vp, vp, vp, vp, sz, sz, sz, sz, fl, it, it, vp]
-    lib.msd_groupnorm_plan.argtypes = [sz, sz, sz, sz, it, it] + [ctypes.POINTER(ctypes.c_int)] * 3
+    lib.msd_groupnorm_plan.argtypes = [sz, sz, sz, sz, it, it, it] + [ctypes.POINTER(ctypes.c_int)] * 4
     lib.msd_layernorm.argtypes = [vp, vp, vp, vp, sz, sz, fl, it, vp]
     lib.msd_geglu.argtypes = [vp, vp, sz, sz, it, vp]
     lib.msd_copy.argtypes = [vp, vp, sz, vp]
@@ -163,11 +163,13 @@ def groupnorm(x, gamma, beta, groups, eps=1e-5, fuse_silu=False, out=None, noall
     return out
 
 
-def groupnorm_plan(batch, channels, hw, groups=32, dtype_code=DTYPE_F16, noalloc=False):
-    """(split, threads, vectors per lane) of the launch msd_groupnorm makes for this shape;
-    (0, 0, 0) = the general kernel.  Host arithmetic, no GPU needed."""
-    out = [ctypes.c_int(0) for _ in range(3)]
-    check(load_library().msd_groupnorm_plan(batch, channels, hw, groups, dtype_code, int(noalloc),
+def groupnorm_plan(batch, channels, hw, groups=32, dtype_code=DTYPE_F16, noalloc=False, in_place=False):
+    """(split, threads, vectors per lane, writers) of the launch msd_groupnorm makes for this
+    shape; (0, 0, 0, 1) = the general kernel; writers > 1 = that many workgroups share each whole
+    (sample, group) and store a part of it each (never for a call in place).  Host arithmetic,
+    no GPU needed."""
+    out = [ctypes.c_int(0) for _ in range(4)]
+    check(load_library().msd_groupnorm_plan(batch, channels, hw, groups, dtype_code, int(noalloc), int(in_place),
                                             *[ctypes.byref(o) for o in out]))
     return tuple(o.value for o in out)
 

@@ -224,6 +224,10 @@ int msd_set_tuning(int knob, int value) {
         case MSD_TUNE_GN_SPIN_LIMIT:
             g_tuning.gn_spin_limit = value;
             return MSD_OK;
+        case MSD_TUNE_GN_WRITERS:
+            if (value && ((value & (value - 1)) != 0 || value > 16)) return MSD_ERR_INVALID_VALUE;
+            g_tuning.gn_writers = value;
+            return MSD_OK;
         default:
             return MSD_ERR_INVALID_VALUE;
     }
@@ -251,19 +255,20 @@ int msd_groupnorm(const void *x, void *y, const float *gamma, const float *beta,
 }
 
 int msd_groupnorm_plan(size_t batch, size_t channels, size_t hw, size_t groups, int dtype, int noalloc,
-                       int *split, int *threads, int *vectors_per_lane) {
-    if (!split || !threads || !vectors_per_lane) return MSD_ERR_INVALID_VALUE;
+                       int in_place, int *split, int *threads, int *vectors_per_lane, int *writers) {
+    if (!split || !threads || !vectors_per_lane || !writers) return MSD_ERR_INVALID_VALUE;
     if (groups == 0 || channels == 0 || channels % groups != 0) return MSD_ERR_INVALID_VALUE;
     if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
     if (batch * groups > 0x7FFFFFFFull || (channels / groups) * hw > 0x7FFFFFFFull) return MSD_ERR_INVALID_VALUE;
     if (noalloc && batch * groups > kStaticUnits) return MSD_ERR_SCRATCH_LIMIT;
-    GnDecision d{0, 0, 0, 0};
+    GnDecision d{0, 0, 0, 0, 1};
     if (batch * hw != 0)
         d = gn_decide(dtype == MSD_DTYPE_F32 ? 4 : 2, batch, channels, hw, groups, true,
-                      noalloc ? (size_t)kStaticUnits : (size_t)kGnMaxUnits);
+                      noalloc ? (size_t)kStaticUnits : (size_t)kGnMaxUnits, in_place == 0);
     *split = (int)d.split;
     *threads = (int)d.threads;
     *vectors_per_lane = (int)d.k;
+    *writers = (int)d.writers;
     return MSD_OK;
 }
 

@@ -53,6 +53,12 @@ struct GnParams {
     float eps;
     float inv_count;         // 1 / elements per unit
     uint32_t spin_limit;     // polls before a slice stops waiting for a sibling's words
+    // gn_slice_kernel<..., SHARED>: `writers` workgroups per whole unit; each loads and reduces the
+    // whole unit and normalises and stores one part of it
+    uint32_t writers;        // power of two
+    uint32_t writers_shift;  // log2(writers)
+    uint32_t part_vecs;      // vectors per part, a multiple of 64 (a wavefront is inside one part or outside)
+    uint32_t same_xcd;       // the writers of a unit have block ids 8 apart: one XCD, one L2 (units % 8 == 0)
 };
 
 // Sum over the workgroup (blockDim.x / 64 wavefronts); one barrier.
@@ -282,11 +288,11 @@ __device__ __forceinline__ void gn_slice_stats(u32x4 (&raw)[K], uint32_t n_valid
 }
 
 // FULL: every lane owns exactly K vectors (no masking anywhere).
-template <typename T, int K, bool SILU, bool FULL>
+template <typename T, int K, bool SILU, bool FULL, bool SHARED>
 __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
                                         const float *__restrict__ gamma,
                                         const float *__restrict__ beta, const GnScratch &scratch,
-                                        const GnParams &p, uint32_t unit, uint32_t slice,
+                                        const GnParams &p, uint32_t unit, uint32_t slice, uint32_t part,
                                         uint32_t v_begin, uint32_t v_end, float *red_a,
                                         float *red_b, float *red_c, float *stats, float2 *aff) {
     constexpr int EPV = Store<T>::EPV;
@@ -297,7 +303,7 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
 
     // launch count of this unit: the tag of this launch's exchange (latency hidden by the loads)
     uint32_t epoch = 0;
-    if (p.split > 1 && tid == 0)
+    if (!SHARED && p.split > 1 && tid == 0)
         epoch = __hip_atomic_load(scratch.epoch + unit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
     // ---- the slice goes into registers.  Lanes past the end of a ragged slice re-read its
@@ -374,7 +380,7 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
 
     float mean, rstd;
     uint32_t arrived_before = 0;
-    if (p.split == 1) {
+    if (SHARED || p.split == 1) {
         mean = slice_mean;
         rstd = __builtin_amdgcn_rsqf(slice_m2 * p.inv_count + p.eps);
     } else {
@@ -428,6 +434,12 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
                     b_next = gb.y;
                 }
             }
+            // several writers per unit: this one normalises and stores the vectors of its part
+            // only; a wavefront is inside a part or outside it as a whole
+            if (SHARED) {  // (decided per wavefront: a scalar branch)
+                const uint32_t first = __builtin_amdgcn_readfirstlane(vidx(k, lane_again()));
+                if (first - part * p.part_vecs >= p.part_vecs) continue;
+            }
             const float a = rstd * g_k;
             const float b_fold = fmaf(-mean, a, b_k);
             float f[EPV];
@@ -450,13 +462,13 @@ __device__ __forceinline__ void gn_body(const T *x, const T *chunk, T *y,
         epilogue(std::true_type{});
     else
         epilogue(std::false_type{});
-    if (p.split > 1 && tid == 0) gn_exchange_close(scratch, p, unit, epoch, arrived_before);
+    if (!SHARED && p.split > 1 && tid == 0) gn_exchange_close(scratch, p, unit, epoch, arrived_before);
 }
 
 // Up to five vectors per lane (four for float storage) the kernel fits 64 registers: eight
 // wavefronts per SIMD, so two 1024-lane workgroups share a CU and one loads while the other
 // computes (what large batches need).
-template <typename T, int K, bool SILU>
+template <typename T, int K, bool SILU, bool SHARED>
 __global__ __launch_bounds__(kGnMaxThreads, (K <= (sizeof(T) == 2 ? 5 : 4) ? 8 : 4)) void gn_slice_kernel(
     const T *x, const T *chunk, T *y, const float *__restrict__ gamma,
     const float *__restrict__ beta, GnScratch scratch, GnParams p) {
@@ -465,17 +477,27 @@ __global__ __launch_bounds__(kGnMaxThreads, (K <= (sizeof(T) == 2 ? 5 : 4) ? 8 :
     __shared__ float red_c[kGnMaxThreads / kWave];
     __shared__ float stats[2];
     __shared__ float2 aff[K <= kGnPrefetchAffineK ? 1 : kGnLdsChannels];  // (gamma, beta) of the group's channels
-    const uint32_t unit = blockIdx.x >> p.split_shift;
-    const uint32_t slice = blockIdx.x & (p.split - 1);
+    uint32_t unit, slice, part;
+    if (SHARED) {  // whole units, `writers` workgroups each
+        const uint32_t j = p.same_xcd ? blockIdx.x >> 3 : blockIdx.x;
+        part = j & (p.writers - 1);
+        unit = j >> p.writers_shift;
+        if (p.same_xcd) unit = (unit << 3) + (blockIdx.x & 7);
+        slice = 0;
+    } else {
+        unit = blockIdx.x >> p.split_shift;
+        slice = blockIdx.x & (p.split - 1);
+        part = 0;
+    }
     const uint32_t v_begin = slice * p.vec_per_slice;
     const uint32_t v_end = min(p.vec_per_unit, v_begin + p.vec_per_slice);
     // uniform over the workgroup; the largest K is only launched on slices it fits exactly
     if (K == kGnMaxK || v_end - v_begin == K * blockDim.x)
-        gn_body<T, K, SILU, true>(x, chunk, y, gamma, beta, scratch, p, unit, slice, v_begin, v_end,
-                                  red_a, red_b, red_c, stats, aff);
+        gn_body<T, K, SILU, true, SHARED>(x, chunk, y, gamma, beta, scratch, p, unit, slice, part, v_begin, v_end,
+                                          red_a, red_b, red_c, stats, aff);
     else
-        gn_body<T, K, SILU, false>(x, chunk, y, gamma, beta, scratch, p, unit, slice, v_begin, v_end,
-                                   red_a, red_b, red_c, stats, aff);
+        gn_body<T, K, SILU, false, SHARED>(x, chunk, y, gamma, beta, scratch, p, unit, slice, part, v_begin, v_end,
+                                           red_a, red_b, red_c, stats, aff);
 }
 
 // Any shape or alignment: one workgroup per unit, three passes over global memory with
@@ -756,16 +778,29 @@ GnPlan plan_slice(uint32_t vecs, uint32_t split, uint32_t force_threads, uint32_
     return pl;
 }
 
+// Kernels with several writers per unit exist up to this many vectors per lane (units of up
+// to 10240 vectors on 1024 lanes).
+constexpr int kGnSharedMaxK = 10;
+
 template <typename T, int K>
-void gn_launch_k(bool silu, uint32_t blocks, uint32_t threads, hipStream_t stream, const T *x,
+void gn_launch_k(bool silu, bool shared, uint32_t blocks, uint32_t threads, hipStream_t stream, const T *x,
                  const T *chunk, T *y, const float *gamma, const float *beta, const GnScratch &sc,
                  const GnParams &p) {
-    if (silu)
-        hipLaunchKernelGGL((gn_slice_kernel<T, K, true>), dim3(blocks), dim3(threads), 0, stream, x,
+    if (K <= kGnSharedMaxK && shared) {
+        constexpr int KS = K <= kGnSharedMaxK ? K : 1;  // (larger K never get here: no such instances)
+        if (silu)
+            hipLaunchKernelGGL((gn_slice_kernel<T, KS, true, true>), dim3(blocks), dim3(threads), 0, stream, x,
+                               chunk, y, gamma, beta, sc, p);
+        else
+            hipLaunchKernelGGL((gn_slice_kernel<T, KS, false, true>), dim3(blocks), dim3(threads), 0, stream,
+                               x, chunk, y, gamma, beta, sc, p);
+    } else if (silu) {
+        hipLaunchKernelGGL((gn_slice_kernel<T, K, true, false>), dim3(blocks), dim3(threads), 0, stream, x,
                            chunk, y, gamma, beta, sc, p);
-    else
-        hipLaunchKernelGGL((gn_slice_kernel<T, K, false>), dim3(blocks), dim3(threads), 0, stream,
+    } else {
+        hipLaunchKernelGGL((gn_slice_kernel<T, K, false, false>), dim3(blocks), dim3(threads), 0, stream,
                            x, chunk, y, gamma, beta, sc, p);
+    }
 }
 
 template <typename T>
@@ -780,13 +815,38 @@ int gn_generic(bool silu, const T *x, const T *chunk, T *y, const float *gamma, 
 
 }  // namespace
 
+// Writers per whole unit when the launch may share units (1: it does not).  A unit's time is
+// its load, its statistics and the epilogue of SiLU and stores, one behind the other on one
+// CU; with w workgroups per unit, each loading and reducing all of it (the copies meet in the
+// L2 of the XCD they share) and finishing a w-th of it, the epilogue and the stores shrink to
+// a w-th while nothing is exchanged.  Best where it gives the chip about one workgroup per CU
+// (measured on every UNet shape, fp16 / fp32, us per launch against the usual plan; 64 units:
+// 2560 vectors 4.76 -> 4.34 (2 writers) -> 4.06 (4) -> 5.07 (8); 5120 vectors, otherwise cut
+// in four with an exchange, 6.00 -> 5.33 (4); 32 units: 2560 vectors 4.59 -> 3.59 (8); 128
+// units: 4.70 (2) against 5.09 and 5.62 (4); 256 units and more: always slower).  Past 5120
+// vectors of 2-byte elements (10240 of 4-byte ones, 5120 with eight writers) the repeated
+// loads cost more than the shorter epilogue gains (7680 vectors, 64 units: 6.71 against 6.56
+// cut in four).
+uint32_t gn_auto_writers(size_t elt, size_t units, size_t vec_per_unit) {
+    // The writers of a unit must run on one XCD (block ids 8 apart: workgroups are dealt to the
+    // XCDs in turn), which needs the units in whole rows of 8; on adjacent blocks, that is on
+    // different XCDs, every copy comes from memory: 5.28 us for the 4.76 above.
+    if (units % 8 != 0) return 1;
+    uint32_t w = 1;
+    while (w < 8 && units * w * 2 <= kChipCus) w *= 2;
+    const size_t limit = (elt == 2 || w >= 8) ? 5120 : 10240;
+    return vec_per_unit <= limit ? w : 1;
+}
+
 // What a GroupNorm launch looks like for a shape: split == 0 means the general kernel (one
 // workgroup per unit, any alignment); otherwise `split` workgroups of `threads` lanes per unit,
 // each holding its slice as `k` vectors per lane.  `elt` = bytes per element, `max_units` = units
-// the exchange scratch has room for.  Reads the tuning knobs.
+// the exchange scratch has room for.  `writers` > 1 (only where `may_share`: the output does
+// not overlap the input) means whole units with that many workgroups each, every one loading and
+// reducing the whole unit and storing its part of it.  Reads the tuning knobs.
 GnDecision gn_decide(size_t elt, size_t batch, size_t channels, size_t hw, size_t groups, bool aligned,
-                     size_t max_units) {
-    GnDecision d{0, 0, 0, 0};
+                     size_t max_units, bool may_share) {
+    GnDecision d{0, 0, 0, 0, 1};
     const size_t epv = 16 / elt;
     const int tune_split = g_tuning.gn_split.load(std::memory_order_relaxed);
     const int tune_threads = g_tuning.gn_threads.load(std::memory_order_relaxed);
@@ -798,6 +858,29 @@ GnDecision gn_decide(size_t elt, size_t batch, size_t channels, size_t hw, size_
 
     const size_t vec_per_unit = unit_size / epv;
     constexpr uint32_t kMaxK = kGnMaxK;
+
+    // ---- several writers per whole unit
+    const int tune_writers = g_tuning.gn_writers.load(std::memory_order_relaxed);
+    if (may_share && tune_split <= 1 && tune_writers != 1 && vec_per_unit <= (size_t)kGnMaxThreads * kGnSharedMaxK) {
+        uint32_t writers = tune_writers > 1 ? (uint32_t)tune_writers : gn_auto_writers(elt, units, vec_per_unit);
+        while (writers > 1 && vec_per_unit < (size_t)writers * kWave) writers /= 2;  // a part is at least a wavefront's vectors
+        if (writers > 1) {
+            uint32_t force = 0;
+            if (tune_threads >= kWave && tune_threads <= kGnMaxThreads && tune_threads % kWave == 0 &&
+                (size_t)tune_threads * kGnSharedMaxK >= vec_per_unit)
+                force = (uint32_t)tune_threads;
+            const GnPlan pl = plan_slice((uint32_t)vec_per_unit, 1, force, kGnSharedMaxK, true, units * writers, elt);
+            if (pl.k != 0 && !(pl.k > kGnPrefetchAffineK && cpg > kGnLdsChannels)) {
+                d.split = 1;
+                d.threads = pl.threads;
+                d.k = (uint32_t)pl.k;
+                d.vec_per_slice = (uint32_t)vec_per_unit;
+                d.writers = writers;
+                return d;
+            }
+        }
+    }
+
     const size_t slice_cap = (size_t)kGnMaxThreads * kGnMaxRaggedK;  // vectors one workgroup can hold
     // smallest power-of-two split whose slices fit in registers
     uint32_t split = 1;
@@ -887,8 +970,13 @@ int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma
     if (units == 0 || unit_size == 0) return MSD_OK;
     if (units > 0x7FFFFFFFull || unit_size > 0x7FFFFFFFull) return MSD_ERR_INVALID_VALUE;
     if (fixed != nullptr && units > fixed->units) return MSD_ERR_SCRATCH_LIMIT;
+    // several workgroups may share a unit only if none of them can store into what another still
+    // loads: the output must lie apart from the input
+    const char *xb = reinterpret_cast<const char *>(x), *yb = reinterpret_cast<const char *>(y);
+    const size_t bytes = units * unit_size * sizeof(T);
+    const bool apart = xb + bytes <= yb || yb + bytes <= xb;
     const GnDecision d = gn_decide(sizeof(T), batch, channels, hw, groups, aligned16(x) && aligned16(y),
-                                   fixed != nullptr ? fixed->units : kGnMaxUnits);
+                                   fixed != nullptr ? fixed->units : kGnMaxUnits, apart);
     if (d.split == 0)
         return gn_generic<T>(silu, x, chunk, y, gamma, beta, units, unit_size, hw, groups, cpg, eps, stream);
 
@@ -904,6 +992,11 @@ int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma
     p.eps = eps;
     p.inv_count = 1.0f / (float)unit_size;
     p.spin_limit = tune_spin > 0 ? (uint32_t)tune_spin : kGnSpinLimit;
+    const bool shared = d.writers > 1;
+    p.writers = d.writers;
+    p.writers_shift = (uint32_t)__builtin_ctz(d.writers);
+    p.part_vecs = (uint32_t)((((p.vec_per_unit + d.writers - 1) / d.writers + kWave - 1) / kWave) * kWave);
+    p.same_xcd = (shared && units % 8 == 0) ? 1u : 0u;
 
     GnScratch sc{nullptr, nullptr, nullptr, nullptr, nullptr, 0};
     if (fixed != nullptr) {
@@ -912,20 +1005,20 @@ int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma
         const hipError_t err = get_scratch(stream, &sc);
         if (err != hipSuccess) return (int)err;
     }
-    const uint32_t blocks = (uint32_t)(units * split);
+    const uint32_t blocks = (uint32_t)(units * split * d.writers);
     const uint32_t threads = d.threads;
     switch (d.k) {
-        case 1: gn_launch_k<T, 1>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
-        case 2: gn_launch_k<T, 2>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
-        case 3: gn_launch_k<T, 3>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
-        case 4: gn_launch_k<T, 4>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
-        case 5: gn_launch_k<T, 5>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
-        case 6: gn_launch_k<T, 6>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
-        case 8: gn_launch_k<T, 8>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
-        case 10: gn_launch_k<T, 10>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
-        case 12: gn_launch_k<T, 12>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
-        case 16: gn_launch_k<T, 16>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
-        case 20: gn_launch_k<T, 20>(silu, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 1: gn_launch_k<T, 1>(silu, shared, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 2: gn_launch_k<T, 2>(silu, shared, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 3: gn_launch_k<T, 3>(silu, shared, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 4: gn_launch_k<T, 4>(silu, shared, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 5: gn_launch_k<T, 5>(silu, shared, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 6: gn_launch_k<T, 6>(silu, shared, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 8: gn_launch_k<T, 8>(silu, shared, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 10: gn_launch_k<T, 10>(silu, shared, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 12: gn_launch_k<T, 12>(silu, shared, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 16: gn_launch_k<T, 16>(silu, shared, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
+        case 20: gn_launch_k<T, 20>(silu, shared, blocks, threads, stream, x, chunk, y, gamma, beta, sc, p); break;
         default: return MSD_ERR_INVALID_VALUE;  // not a K the kernels are built for: a planning error
     }
     return launch_status();
@@ -1000,6 +1093,10 @@ int gn_tokens_dispatch(const void *xv, void *yv, const float *gamma, const float
     q.base.vec_per_slice = (uint32_t)nvec;
     q.base.split = split;
     q.base.split_shift = (uint32_t)__builtin_ctz(split);
+    q.base.writers = 1;
+    q.base.writers_shift = 0;
+    q.base.part_vecs = 0;
+    q.base.same_xcd = 0;
     q.base.groups = (uint32_t)groups;
     q.base.ch_per_group = (uint32_t)cpg;
     q.base.hw_vec = make_fast_div((uint32_t)hw_vec);

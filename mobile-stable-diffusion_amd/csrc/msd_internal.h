@@ -36,6 +36,7 @@ hipError_t get_static_scratch(GnScratch *out);
 struct Tuning {
     std::atomic<int> gn_split{0};
     std::atomic<int> gn_threads{0};
+    std::atomic<int> gn_writers{0};
     std::atomic<int> ln_chunk{0};
     std::atomic<int> ln_threads{0};
     std::atomic<int> geglu_vectors{0};
@@ -53,9 +54,10 @@ struct GnDecision {
     uint32_t threads;
     uint32_t k;
     uint32_t vec_per_slice;
+    uint32_t writers;  // workgroups per whole unit that each store a part of it (1: the usual launch)
 };
 GnDecision gn_decide(size_t elt, size_t batch, size_t channels, size_t hw, size_t groups, bool aligned,
-                     size_t max_units);
+                     size_t max_units, bool may_share);
 
 // ---- per-dtype dispatchers (T = float or __half), defined in the kernel files ----
 // fixed: scratch to use instead of the stream's own (units beyond its capacity are refused)

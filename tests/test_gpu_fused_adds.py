@@ -57,10 +57,16 @@ def test_chunk_add_groupnorm_equals_two_launches(msd, orc, cuda, shape, groups, 
     tmp = msd.chunkwise_add(xd, ed, hw)
     two = msd.groupnorm(tmp, gd, bd, groups, 1e-5, True)
     assert torch.equal(fused, two)
-    # in place, as the reference runs its out-norm (M/nn/ResBlock.cpp:222)
-    inplace = msd.chunk_add_groupnorm(xd.clone(), ed, gd, bd, groups, 1e-5, True)
+    # in place, as the reference runs its out-norm (M/nn/ResBlock.cpp:222): the launch never lets
+    # several workgroups share a unit then, so it is compared with the same launch out of place
+    lib = msd.load_library()
+    assert lib.msd_set_tuning(msd.TUNE_GN_WRITERS, 1) == 0
+    try:
+        apart = msd.chunk_add_groupnorm(xd.clone(), ed, gd, bd, groups, 1e-5, True)
+    finally:
+        assert lib.msd_set_tuning(msd.TUNE_GN_WRITERS, 0) == 0
     xc = xd.clone()
-    assert torch.equal(msd.chunk_add_groupnorm(xc, ed, gd, bd, groups, 1e-5, True, out=xc), inplace)
+    assert torch.equal(msd.chunk_add_groupnorm(xc, ed, gd, bd, groups, 1e-5, True, out=xc), apart)
     # oracle: chunkwise_add, (storage rounding), group norm, silu
     s = orc.chunkwise_add(xin, ein, hw)
     if half:

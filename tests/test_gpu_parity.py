@@ -53,7 +53,18 @@ def _run_groupnorm(msd, orc, cuda, x, g, b, groups, eps, silu, half, inplace=Fal
 
 
 # ----------------------------------------------------------------- GroupNorm
-def test_config1_groupnorm_silu_fp32(msd, orc, cuda):
+@pytest.fixture(params=[0, 1], ids=["writers-auto", "one-writer"])
+def gn_writers(request, msd):
+    """Runs a test twice: with the launch plan free to let several workgroups share a whole
+    (sample, group) when the output lies apart from the input, and with that switched off (one
+    workgroup per unit or slices with an exchange, as for a call in place)."""
+    lib = msd.load_library()
+    assert lib.msd_set_tuning(msd.TUNE_GN_WRITERS, request.param) == 0
+    yield request.param
+    assert lib.msd_set_tuning(msd.TUNE_GN_WRITERS, 0) == 0
+
+
+def test_config1_groupnorm_silu_fp32(msd, orc, cuda, gn_writers):
     x = orc.normal((1, 320, 64, 64), seed=1001)
     g, b = _affine(orc, 320, 1001)
     _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half=False)
@@ -62,7 +73,7 @@ def test_config1_groupnorm_silu_fp32(msd, orc, cuda):
 
 @pytest.mark.parametrize("half", [False, True], ids=["f32", "f16"])
 @pytest.mark.parametrize("channels,hw,seed", CFG2_SHAPES)
-def test_config2_groupnorm_silu_sweep(msd, orc, cuda, channels, hw, seed, half):
+def test_config2_groupnorm_silu_sweep(msd, orc, cuda, channels, hw, seed, half, gn_writers):
     side = int(round(hw ** 0.5))
     x = orc.normal((2, channels, side, side), seed=seed, sigma=2.0)
     g, b = _affine(orc, channels, seed)
@@ -73,14 +84,14 @@ def test_config2_groupnorm_silu_sweep(msd, orc, cuda, channels, hw, seed, half):
 
 
 @pytest.mark.parametrize("channels,hw", UNET_GN_SHAPES)
-def test_unet_step_groupnorm_shapes_fp16(msd, orc, cuda, channels, hw):
+def test_unet_step_groupnorm_shapes_fp16(msd, orc, cuda, channels, hw, gn_writers):
     x = orc.normal((2, channels, hw), seed=5001 + channels + hw, sigma=1.5, mean=0.2)
     g, b = _affine(orc, channels, 5001 + channels)
     _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half=True)
 
 
 @pytest.mark.parametrize("half", [False, True], ids=["f32", "f16"])
-def test_groupnorm_in_place_and_no_silu(msd, orc, cuda, half):
+def test_groupnorm_in_place_and_no_silu(msd, orc, cuda, half, gn_writers):
     # in place as at M/nn/ResBlock.cpp:222; eps 1e-6 without SiLU as in SpatialTransformer
     x = orc.normal((2, 640, 32, 32), seed=77, sigma=1.0, mean=-0.5)
     g, b = _affine(orc, 640, 77)
@@ -153,12 +164,12 @@ def test_groupnorm_large_batch_plan_and_wide_groups(msd, orc, cuda):
     lib = msd.load_library()
     x = orc.normal((17, 320, 64, 64), seed=521, sigma=1.2, mean=-0.3)
     g, b = _affine(orc, 320, 521)
-    assert msd.groupnorm_plan(17, 320, 4096) == (1, 256, 20)
+    assert msd.groupnorm_plan(17, 320, 4096) == (1, 256, 20, 1)
     _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, True)
     _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, False)
     # the other unit sizes of the UNet at that batch: 10 and 5 vectors per lane, ragged 16 and 8
-    for channels, hw, plan in ((640, 1024, (1, 256, 10)), (1280, 256, (1, 256, 5)), (960, 1024, (1, 256, 16)),
-                               (1920, 256, (1, 256, 8))):
+    for channels, hw, plan in ((640, 1024, (1, 256, 10, 1)), (1280, 256, (1, 256, 5, 1)), (960, 1024, (1, 256, 16, 1)),
+                               (1920, 256, (1, 256, 8, 1))):
         assert msd.groupnorm_plan(17, channels, hw) == plan
         xs = orc.normal((17, channels, hw), seed=523 + channels, sigma=1.4, mean=0.2)
         gs, bs = _affine(orc, channels, 523 + channels)
@@ -242,7 +253,7 @@ def test_groupnorm_slice_that_stops_waiting_computes_its_siblings_statistics(msd
     assert msd.gn_fallbacks() > 0  # the path was really taken
     # back to the normal limit: no workgroup gives up on an idle GPU
     msd.gn_fallbacks(reset=True)
-    _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, True)
+    _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, True, inplace=True)
     assert msd.gn_fallbacks() == 0
     assert msd.status() == 0
 
@@ -272,7 +283,7 @@ def test_groupnorm_repeated_launches_reuse_scratch(msd, orc, cuda):
     ((1, 4, 512, 512), 1),    # one huge group: maximum split
 ])
 @pytest.mark.parametrize("half", [False, True], ids=["f32", "f16"])
-def test_groupnorm_edge_shapes(msd, orc, cuda, shape, groups, half):
+def test_groupnorm_edge_shapes(msd, orc, cuda, shape, groups, half, gn_writers):
     x = orc.normal(shape, seed=sum(shape), sigma=1.3, mean=0.1)
     xin = orc.round_to_half(x) if half else x
     g, b = _affine(orc, shape[1], 31)
@@ -322,7 +333,7 @@ def test_groupnorm_statistics_property_full_size(msd, orc, cuda):
 
 @pytest.mark.parametrize("mean,sigma", [(5.0, 1.0), (50.0, 1.0), (500.0, 1.0), (1.0, 0.01), (100.0, 0.01),
                                         (1e4, 10.0), (0.0, 1e-4)])
-def test_groupnorm_ill_conditioned_inputs_track_float64_like_the_reference(msd, orc, cuda, mean, sigma):
+def test_groupnorm_ill_conditioned_inputs_track_float64_like_the_reference(msd, orc, cuda, mean, sigma, gn_writers):
     """With |mean| >> sigma float32 itself cannot hold 1e-5 (the reference's two-pass algorithm is
     1e-4 .. 1e-3 away from float64 there).  The kernel must then be no further from float64
     than that restatement is (it is closer: centred statistics per wavefront, Chan merges)."""
@@ -623,7 +634,7 @@ def test_groupnorm_two_streams_have_private_scratch(msd, orc, cuda):
 
 
 @pytest.mark.parametrize("batch,channels,hw", [(8, 320, 4096), (4, 640, 4096), (8, 960, 1024), (5, 320, 4096)])
-def test_groupnorm_larger_batches_pick_other_splits(msd, orc, cuda, batch, channels, hw):
+def test_groupnorm_larger_batches_pick_other_splits(msd, orc, cuda, batch, channels, hw, gn_writers):
     # 128 / 256 units: the launch plan cuts units in two or not at all instead of in four
     x = orc.normal((batch, channels, hw), seed=batch * 1000 + channels, sigma=1.5, mean=0.2)
     g, b = _affine(orc, channels, 77)
@@ -633,20 +644,84 @@ def test_groupnorm_larger_batches_pick_other_splits(msd, orc, cuda, batch, chann
 
 
 @pytest.mark.parametrize("batch,channels,hw,plan", [
-    (1, 320, 4096, (4, 640, 4)), (1, 640, 1024, (4, 640, 2)), (1, 960, 4096, (8, 960, 4)),
-    (2, 960, 4096, (8, 960, 4)), (2, 320, 4096, (2, 1024, 5)), (2, 1920, 256, (1, 960, 4)),
-    (2, 640, 256, (1, 640, 2)), (4, 640, 4096, (4, 512, 10)), (4, 1920, 1024, (4, 960, 4)),
-    (8, 320, 4096, (2, 512, 10)), (8, 640, 4096, (2, 512, 20))])
+    (1, 320, 4096, (4, 640, 4, 1)), (1, 640, 1024, (4, 640, 2, 1)), (1, 960, 4096, (8, 960, 4, 1)),
+    (2, 960, 4096, (8, 960, 4, 1)), (2, 320, 4096, (2, 1024, 5, 1)), (2, 1920, 256, (1, 960, 4, 1)),
+    (2, 640, 256, (1, 640, 2, 1)), (4, 640, 4096, (4, 512, 10, 1)), (4, 1920, 1024, (4, 960, 4, 1)),
+    (8, 320, 4096, (2, 512, 10, 1)), (8, 640, 4096, (2, 512, 20, 1))])
 def test_groupnorm_fp32_plans_at_unet_shapes(msd, orc, cuda, batch, channels, hw, plan):
-    """4-byte elements are cut more often and into exact fits of up to four vectors per lane."""
-    assert msd.groupnorm_plan(batch, channels, hw, 32, msd.DTYPE_F32) == plan
+    """4-byte elements are cut more often and into exact fits of up to four vectors per lane (the
+    plans of a call in place, which is how the tensor is run here)."""
+    assert msd.groupnorm_plan(batch, channels, hw, 32, msd.DTYPE_F32, in_place=True) == plan
     x = orc.normal((batch, channels, hw), seed=batch * 1000 + channels + hw, sigma=2.0, mean=-0.1)
     g, b = _affine(orc, channels, 78)
-    _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half=False)
+    _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half=False, inplace=True)
     assert msd.status() == 0
 
 
-def test_groupnorm_many_units_and_register_limits(msd, orc, cuda):
+@pytest.mark.parametrize("writers", [2, 4, 8, 16])
+def test_groupnorm_several_writers_per_unit_give_the_bits_of_one(msd, orc, cuda, writers):
+    """Several workgroups per whole (sample, group), each loading and reducing all of it and storing
+    one part: the statistics are computed as by a single workgroup, so the output must be the same
+    bit for bit - for full and ragged units, either element size, with and without SiLU, with the
+    embedding addend, for units in whole rows of 8 (writers 8 blocks apart) and not (adjacent) -
+    and a call in place must not take that launch at all."""
+    torch = _torch()
+    lib = msd.load_library()
+    cases = [((2, 320, 64, 64), 32), ((2, 640, 32, 32), 32), ((1, 96, 24, 24), 32), ((3, 24, 40, 40), 3),
+             ((2, 1280, 8, 8), 32), ((1, 64, 56, 72), 8), ((5, 32, 40, 40), 4), ((2, 960, 32, 32), 32)]
+    try:
+        for shape, groups in cases:
+            for half in (True, False):
+                channels = shape[1]
+                x = orc.normal(shape, seed=sum(shape) + writers, sigma=1.8, mean=0.4)
+                xin = orc.round_to_half(x) if half else x
+                g, b = _affine(orc, channels, 83)
+                emb = orc.normal((shape[0], channels), seed=84, sigma=0.5)
+                emb = orc.round_to_half(emb) if half else emb
+                xd, gd, bd, ed = _to_dev(xin, cuda, half), _to_dev(g, cuda), _to_dev(b, cuda), _to_dev(emb, cuda, half)
+                hw = shape[2] * shape[3]
+                code = msd.DTYPE_F16 if half else msd.DTYPE_F32
+                # the same whole-unit launch (same lanes, same vectors per lane) with one writer
+                assert lib.msd_set_tuning(msd.TUNE_GN_SPLIT, 1) == 0
+                assert lib.msd_set_tuning(msd.TUNE_GN_WRITERS, writers) == 0
+                plan = msd.groupnorm_plan(shape[0], channels, hw, groups, code)
+                assert plan[0] == 1 and plan[3] > 1, (shape, half, plan)
+                assert msd.groupnorm_plan(shape[0], channels, hw, groups, code, in_place=True)[3] == 1
+                assert lib.msd_set_tuning(msd.TUNE_GN_THREADS, plan[1]) == 0
+                for silu in (True, False):
+                    assert lib.msd_set_tuning(msd.TUNE_GN_WRITERS, 1) == 0
+                    assert msd.groupnorm_plan(shape[0], channels, hw, groups, code) == plan[:3] + (1,)
+                    one = msd.groupnorm(xd, gd, bd, groups, 1e-5, silu)
+                    one_add = msd.chunk_add_groupnorm(xd, ed, gd, bd, groups, 1e-5, silu)
+                    assert lib.msd_set_tuning(msd.TUNE_GN_WRITERS, writers) == 0
+                    got = msd.groupnorm(xd, gd, bd, groups, 1e-5, silu)
+                    got_add = msd.chunk_add_groupnorm(xd, ed, gd, bd, groups, 1e-5, silu)
+                    assert torch.equal(got, one) and torch.equal(got_add, one_add), (shape, half, silu, plan)
+                    z = xd.clone()
+                    msd.groupnorm(z, gd, bd, groups, 1e-5, silu, out=z)   # in place: one writer
+                    assert torch.equal(z, one), (shape, half, silu, "in place")
+                assert lib.msd_set_tuning(msd.TUNE_GN_THREADS, 0) == 0
+                assert lib.msd_set_tuning(msd.TUNE_GN_SPLIT, 0) == 0
+                ref = orc.groupnorm(xin, g, b, groups, 1e-5, False)
+                if half:
+                    assert_close_f16(got.float().cpu().numpy(), ref, "gn writers f16 %s" % (shape,))
+                else:
+                    assert_close_f32(got.cpu().numpy(), ref, what="gn writers f32 %s" % (shape,))
+    finally:
+        assert lib.msd_set_tuning(msd.TUNE_GN_WRITERS, 0) == 0
+        assert lib.msd_set_tuning(msd.TUNE_GN_THREADS, 0) == 0
+        assert lib.msd_set_tuning(msd.TUNE_GN_SPLIT, 0) == 0
+    # the knob is followed as far as every writer still owns a wavefront's vectors
+    assert lib.msd_set_tuning(msd.TUNE_GN_WRITERS, writers) == 0
+    try:
+        assert msd.groupnorm_plan(2, 320, 4096, 32, msd.DTYPE_F16)[3] == writers
+        assert msd.groupnorm_plan(2, 1280, 64, 32, msd.DTYPE_F16)[3] == min(writers, 4)   # 320 vectors: parts of 64 at least
+    finally:
+        assert lib.msd_set_tuning(msd.TUNE_GN_WRITERS, 0) == 0
+    assert msd.status() == 0
+
+
+def test_groupnorm_many_units_and_register_limits(msd, orc, cuda, gn_writers):
     # more units than scratch slots (never split), and float units that need a split to fit
     for shape, groups, half in [((300, 64, 4, 8), 32, True),     # 9600 units
                                 ((1, 32, 64, 64), 2, False),     # 65536-element float units

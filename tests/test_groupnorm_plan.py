@@ -3,7 +3,8 @@
 A kernel that does not match its launch faults the GPU, so what the planner may hand to the
 register kernel is pinned here: the vectors-per-lane values the kernels are built for, workgroup
 sizes in whole wavefronts, slices that fit their workgroup and own at least one vector, the largest
-vectors-per-lane value only on exact fits, power-of-two slice counts within the exchange scratch.
+vectors-per-lane value only on exact fits, power-of-two slice counts within the exchange scratch,
+several writers only on whole units of at most 10 vectors per lane and never for a call in place.
 The reference has no counterpart: its geometry is fixed (M/nn/GroupNorm.cpp:105-128)."""
 import importlib
 import random
@@ -16,14 +17,14 @@ K_VALUES = {1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 20}
 MAX_SPLIT, MAX_UNITS, STATIC_UNITS = 64, 8192, 1024
 
 
-def _check(batch, channels, hw, groups, code, noalloc=False):
-    split, threads, k = msd.groupnorm_plan(batch, channels, hw, groups, code, noalloc)
+def _check(batch, channels, hw, groups, code, noalloc=False, in_place=False):
+    split, threads, k, writers = msd.groupnorm_plan(batch, channels, hw, groups, code, noalloc, in_place)
     elt = 4 if code == msd.DTYPE_F32 else 2
     epv = 16 // elt
     unit = channels // groups * hw
     if split == 0:
-        assert threads == 0 and k == 0
-        return split, threads, k
+        assert threads == 0 and k == 0 and writers == 1
+        return split, threads, k, writers
     assert hw % epv == 0 and unit * elt < 2 ** 32          # what the register kernel assumes
     vecs = unit // epv
     assert split & (split - 1) == 0 and 1 <= split <= MAX_SPLIT
@@ -39,50 +40,70 @@ def _check(batch, channels, hw, groups, code, noalloc=False):
         assert per_slice * split == vecs and per_slice == 20 * threads
     if k > 6:                                              # gamma / beta of the group go through LDS
         assert channels // groups <= 1024
-    return split, threads, k
+    assert writers in (1, 2, 4, 8, 16)
+    if writers > 1:                                        # whole units, kernels built up to K = 10,
+        assert split == 1 and k <= 10 and not in_place     # every writer owns a wavefront's vectors at least
+        assert vecs >= writers * 64
+    return split, threads, k, writers
 
 
 def test_plans_of_the_unet_shapes_at_batch_2_and_32():
     f16, f32 = msd.DTYPE_F16, msd.DTYPE_F32
-    expected = {
-        (2, 320, 4096, f16): (4, 640, 2), (2, 640, 1024, f16): (1, 512, 5), (2, 1280, 256, f16): (1, 512, 3),
-        (2, 1280, 64, f16): (1, 320, 1), (2, 960, 1024, f16): (2, 960, 2), (2, 1920, 256, f16): (1, 960, 2),
-        (1, 320, 4096, f32): (4, 640, 4), (1, 640, 4096, f16): (4, 1024, 3), (1, 960, 4096, f16): (8, 960, 2),
-        (2, 960, 4096, f32): (8, 960, 4), (2, 640, 1024, f32): (1, 1024, 5), (1, 640, 1024, f32): (4, 640, 2),
-        (4, 640, 4096, f32): (4, 512, 10), (8, 640, 4096, f32): (2, 512, 20), (2, 640, 256, f32): (1, 640, 2),
-        (32, 320, 4096, f16): (1, 256, 20), (32, 640, 1024, f16): (1, 256, 10), (32, 1280, 256, f16): (1, 256, 5),
-        (8, 320, 4096, f16): (1, 1024, 5), (32, 960, 4096, f16): (4, 256, 16),
+    # a call in place (the reference's out-norms): one workgroup per unit or slices with an exchange
+    in_place = {
+        (2, 320, 4096, f16): (4, 640, 2, 1), (2, 640, 1024, f16): (1, 512, 5, 1), (2, 1280, 256, f16): (1, 512, 3, 1),
+        (2, 1280, 64, f16): (1, 320, 1, 1), (2, 960, 1024, f16): (2, 960, 2, 1), (2, 1920, 256, f16): (1, 960, 2, 1),
+        (1, 320, 4096, f32): (4, 640, 4, 1), (1, 640, 4096, f16): (4, 1024, 3, 1), (1, 960, 4096, f16): (8, 960, 2, 1),
+        (2, 960, 4096, f32): (8, 960, 4, 1), (2, 640, 1024, f32): (1, 1024, 5, 1), (1, 640, 1024, f32): (4, 640, 2, 1),
+        (4, 640, 4096, f32): (4, 512, 10, 1), (8, 640, 4096, f32): (2, 512, 20, 1), (2, 640, 256, f32): (1, 640, 2, 1),
+        (32, 320, 4096, f16): (1, 256, 20, 1), (32, 640, 1024, f16): (1, 256, 10, 1), (32, 1280, 256, f16): (1, 256, 5, 1),
+        (8, 320, 4096, f16): (1, 1024, 5, 1), (32, 960, 4096, f16): (4, 256, 16, 1),
     }
-    for (batch, channels, hw, code), want in expected.items():
+    for (batch, channels, hw, code), want in in_place.items():
+        assert _check(batch, channels, hw, 32, code, in_place=True) == want, (batch, channels, hw, code)
+    # output apart from the input: up to 256 workgroups share whole units of up to 5120 vectors
+    # (10240 of 4-byte elements with up to four writers); larger units and batches plan as above
+    apart = {
+        (2, 320, 4096, f16): (1, 1024, 5, 4), (2, 640, 1024, f16): (1, 512, 5, 4), (2, 1280, 256, f16): (1, 512, 3, 4),
+        (2, 1280, 64, f16): (1, 320, 1, 4), (2, 960, 1024, f16): (1, 1024, 4, 4), (2, 1920, 256, f16): (1, 960, 2, 4),
+        (2, 1920, 1024, f16): (4, 960, 2, 1), (2, 640, 4096, f16): (4, 1024, 3, 1),
+        (1, 320, 4096, f16): (1, 1024, 5, 8), (1, 1280, 64, f16): (1, 320, 1, 4), (4, 640, 1024, f16): (1, 512, 5, 2),
+        (1, 320, 4096, f32): (4, 640, 4, 1), (1, 640, 1024, f32): (1, 1024, 5, 8), (2, 320, 4096, f32): (1, 1024, 10, 4),
+        (2, 960, 1024, f32): (1, 1024, 8, 4), (2, 960, 4096, f32): (8, 960, 4, 1),
+        (8, 320, 4096, f16): (1, 1024, 5, 1), (32, 320, 4096, f16): (1, 256, 20, 1),
+    }
+    for (batch, channels, hw, code), want in apart.items():
         assert _check(batch, channels, hw, 32, code) == want, (batch, channels, hw, code)
+    assert _check(3, 24, 4096, 3, f16)[3] == 1    # 9 units: not in whole rows of 8, the writers would sit on different XCDs
 
 
 def test_shapes_the_register_kernel_cannot_take_go_to_the_general_kernel():
-    assert msd.groupnorm_plan(2, 320, 4090, 32, msd.DTYPE_F16) == (0, 0, 0)      # hw not in whole vectors
-    assert msd.groupnorm_plan(2, 320, 4094, 32, msd.DTYPE_F32) == (0, 0, 0)
+    assert msd.groupnorm_plan(2, 320, 4090, 32, msd.DTYPE_F16) == (0, 0, 0, 1)   # hw not in whole vectors
+    assert msd.groupnorm_plan(2, 320, 4094, 32, msd.DTYPE_F32) == (0, 0, 0, 1)
     assert msd.groupnorm_plan(1, 32 * 1100, 32, 32, msd.DTYPE_F16)[2] <= 6         # wide groups: no LDS affine
-    assert msd.groupnorm_plan(0, 320, 4096, 32, msd.DTYPE_F16) == (0, 0, 0)        # nothing to do
+    assert msd.groupnorm_plan(0, 320, 4096, 32, msd.DTYPE_F16) == (0, 0, 0, 1)     # nothing to do
     lib = msd.load_library()
     import ctypes
-    o = [ctypes.c_int(7) for _ in range(3)]
+    o = [ctypes.c_int(7) for _ in range(4)]
     refs = [ctypes.byref(v) for v in o]
-    assert lib.msd_groupnorm_plan(2, 320, 4096, 0, msd.DTYPE_F16, 0, *refs) == 1   # no groups
-    assert lib.msd_groupnorm_plan(2, 321, 4096, 32, msd.DTYPE_F16, 0, *refs) == 1  # channels % groups
-    assert lib.msd_groupnorm_plan(2, 320, 4096, 32, 5, 0, *refs) == 1              # unknown dtype
-    assert lib.msd_groupnorm_plan(2, 320, 4096, 32, msd.DTYPE_F16, 0, None, None, None) == 1
-    assert lib.msd_groupnorm_plan(33, 320, 4096, 32, msd.DTYPE_F16, 1, *refs) == -2  # beyond the fixed scratch
+    assert lib.msd_groupnorm_plan(2, 320, 4096, 0, msd.DTYPE_F16, 0, 0, *refs) == 1   # no groups
+    assert lib.msd_groupnorm_plan(2, 321, 4096, 32, msd.DTYPE_F16, 0, 0, *refs) == 1  # channels % groups
+    assert lib.msd_groupnorm_plan(2, 320, 4096, 32, 5, 0, 0, *refs) == 1              # unknown dtype
+    assert lib.msd_groupnorm_plan(2, 320, 4096, 32, msd.DTYPE_F16, 0, 0, None, None, None, None) == 1
+    assert lib.msd_groupnorm_plan(33, 320, 4096, 32, msd.DTYPE_F16, 1, 0, *refs) == -2  # beyond the fixed scratch
 
 
 @pytest.mark.parametrize("seed", range(6))
 def test_random_shapes_always_get_a_launch_that_fits(seed):
     rng = random.Random(seed)
     lib = msd.load_library()
-    knobs = [(0, 0)] + [(rng.choice([0, 1, 2, 4, 8, 16, 32, 64]), rng.choice([0, 64, 128, 256, 320, 512, 640, 768, 1024]))
-                        for _ in range(3)]
+    knobs = [(0, 0, 0)] + [(rng.choice([0, 1, 2, 4, 8, 16, 32, 64]), rng.choice([0, 64, 128, 256, 320, 512, 640, 768, 1024]),
+                            rng.choice([0, 0, 1, 2, 4, 8, 16])) for _ in range(4)]
     try:
-        for split_knob, threads_knob in knobs:
+        for split_knob, threads_knob, writers_knob in knobs:
             assert lib.msd_set_tuning(msd.TUNE_GN_SPLIT, split_knob) == 0
             assert lib.msd_set_tuning(msd.TUNE_GN_THREADS, threads_knob) == 0
+            assert lib.msd_set_tuning(msd.TUNE_GN_WRITERS, writers_knob) == 0
             for _ in range(1500):
                 groups = rng.choice([1, 2, 8, 32, 32, 32, 64])
                 cpg = rng.choice([1, 2, 3, 5, 10, 20, 30, 40, 60, 80, 128, 1100])
@@ -91,7 +112,9 @@ def test_random_shapes_always_get_a_launch_that_fits(seed):
                 code = rng.choice([msd.DTYPE_F16, msd.DTYPE_F32])
                 if cpg * hw > 0x7FFFFFFF or batch * groups > 0x7FFFFFFF:
                     continue
-                _check(batch, groups * cpg, hw, groups, code, noalloc=batch * groups <= STATIC_UNITS and rng.random() < 0.3)
+                _check(batch, groups * cpg, hw, groups, code, noalloc=batch * groups <= STATIC_UNITS and rng.random() < 0.3,
+                       in_place=rng.random() < 0.3)
     finally:
         lib.msd_set_tuning(msd.TUNE_GN_SPLIT, 0)
         lib.msd_set_tuning(msd.TUNE_GN_THREADS, 0)
+        lib.msd_set_tuning(msd.TUNE_GN_WRITERS, 0)
