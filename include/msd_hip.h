@@ -101,7 +101,10 @@ int msd_set_tuning(int knob, int value);
  * the separate silu enqueue that follows it (M/nn/ResBlock.cpp:136-142,
  * K/util.cl:124-134).  Biased variance, y = fma((x-mean)/sqrt(var+eps), gamma[c],
  * beta[c]).  x and y are [batch, channels, hw]; y may alias x exactly (in place,
- * M/nn/ResBlock.cpp:222).  Requires channels % groups == 0.
+ * M/nn/ResBlock.cpp:222).  Requires channels % groups == 0.  When y lies apart from x
+ * and there are fewer than 256 (sample, group) units, several workgroups share each unit
+ * (msd_groupnorm_plan tells); the statistics are then summed in another order than for the
+ * call in place, so the two results can differ in the last bit.
  */
 int msd_groupnorm(const void *x, void *y, const float *gamma, const float *beta,
                   size_t batch, size_t channels, size_t hw, size_t groups, float eps,
