@@ -553,9 +553,14 @@ struct GnTokParams {
     uint32_t channels;
     uint32_t pitch;       // LDS elements between channels: positions per slice + 16 bytes
     FastDiv combos;       // batch * split: (sample, slice) pairs, the fastest part of the block id
+    FastDiv part_len;     // SHARED: vectors of one part, ch_per_group * pos_vecs.d (a multiple of 64)
 };
 
-template <typename T, int K>
+// SHARED: `writers` workgroups per whole unit (output apart from the input by construction).  Each
+// loads and reduces the whole unit, enumerated part by part (a part = all channels over a range of
+// positions, what a slice is above), and normalises, transposes and stores its own part; nothing
+// is exchanged.  The writers of a unit have block ids 8 apart (one XCD: their loads meet in its L2).
+template <typename T, int K, bool SHARED>
 __global__ __launch_bounds__(kGnMaxThreads) void gn_tokens_kernel(
     const T *__restrict__ x, T *__restrict__ y, const float *__restrict__ gamma,
     const float *__restrict__ beta, GnScratch scratch, GnTokParams q) {
@@ -573,27 +578,40 @@ __global__ __launch_bounds__(kGnMaxThreads) void gn_tokens_kernel(
     // that differ by multiples of batch * split, so with workgroups dealt round-robin to the
     // 8 XCDs they meet in one L2 when that product is a multiple of 8 (batch 2 x 4 slices);
     // the slices of a unit stay adjacent
-    const uint32_t group = fast_div(blockIdx.x, q.combos);
-    const uint32_t combo = blockIdx.x - group * q.combos.d;
-    const uint32_t unit = (combo >> p.split_shift) * p.groups + group;
-    const uint32_t slice = combo & (p.split - 1);
-    const uint32_t nvec = p.vec_per_slice;
+    uint32_t unit, slice;  // SHARED: `slice` is the part this workgroup stores
+    if (SHARED) {
+        const uint32_t j = p.same_xcd ? blockIdx.x >> 3 : blockIdx.x;
+        slice = j & (p.writers - 1);
+        unit = j >> p.writers_shift;
+        if (p.same_xcd) unit = (unit << 3) + (blockIdx.x & 7);
+    } else {
+        const uint32_t group = fast_div(blockIdx.x, q.combos);
+        const uint32_t combo = blockIdx.x - group * q.combos.d;
+        unit = (combo >> p.split_shift) * p.groups + group;
+        slice = combo & (p.split - 1);
+    }
+    const uint32_t nvec = SHARED ? p.vec_per_unit : p.vec_per_slice;  // vectors this workgroup holds
     const uint32_t pvs = q.pos_vecs.d;
     const u32x4 *xin = reinterpret_cast<const u32x4 *>(x) + (size_t)unit * p.vec_per_unit;
 
     uint32_t epoch = 0;
-    if (p.split > 1 && tid == 0)
+    if (!SHARED && p.split > 1 && tid == 0)
         epoch = __hip_atomic_load(scratch.epoch + unit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
-    // lane-local vector -> (channel of the group, position vector of the slice)
+    // lane-local vector -> (part, channel of the group, position vector of the part / slice)
     u32x4 raw[K];
     uint32_t cl[K], pv[K];
 #pragma unroll
     for (int k = 0; k < K; k++) {
-        const uint32_t vl = min(k * nt + tid, nvec - 1);  // ragged tail re-reads the last vector
+        uint32_t vl = min(k * nt + tid, nvec - 1);  // ragged tail re-reads the last vector
+        uint32_t part_of = slice;
+        if (SHARED) {
+            part_of = fast_div(vl, q.part_len);
+            vl -= part_of * q.part_len.d;
+        }
         cl[k] = fast_div(vl, q.pos_vecs);
         pv[k] = vl - cl[k] * pvs;
-        raw[k] = load_stream(xin + (size_t)cl[k] * p.hw_vec.d + slice * pvs + pv[k]);
+        raw[k] = load_stream(xin + (size_t)cl[k] * p.hw_vec.d + part_of * pvs + pv[k]);
         const bool have = k * nt + tid < nvec;  // lanes past the end hold zeros (the statistics rely on it)
 #pragma unroll
         for (int i = 0; i < 4; i++) raw[k][i] = have ? raw[k][i] : 0u;
@@ -604,7 +622,7 @@ __global__ __launch_bounds__(kGnMaxThreads) void gn_tokens_kernel(
     gn_slice_stats<T, K, false>(raw, nvec, red_a, red_b, red_c, slice_mean, slice_m2);
 
     float mean, rstd;
-    if (p.split == 1) {
+    if (SHARED || p.split == 1) {
         mean = slice_mean;
         rstd = __builtin_amdgcn_rsqf(slice_m2 * p.inv_count + p.eps);
     } else {
@@ -622,6 +640,10 @@ __global__ __launch_bounds__(kGnMaxThreads) void gn_tokens_kernel(
     T *lds = reinterpret_cast<T *>(lds_vec);
 #pragma unroll
     for (int k = 0; k < K; k++) {
+        if (SHARED) {  // a wavefront lies inside one part (part_len is a multiple of 64): a scalar branch
+            const uint32_t first = __builtin_amdgcn_readfirstlane(min(k * nt + tid, nvec - 1));
+            if (first - slice * q.part_len.d >= q.part_len.d) continue;
+        }
         if (k * nt + tid < nvec) {
             const float a = rstd * gamma[ch0 + cl[k]];
             const float b = beta[ch0 + cl[k]];
@@ -635,7 +657,7 @@ __global__ __launch_bounds__(kGnMaxThreads) void gn_tokens_kernel(
     __syncthreads();
     // the slice counts itself done here, behind the last barrier: nothing waits for the answer
     uint32_t arrived_before = 0;
-    if (p.split > 1 && tid == 0) arrived_before = gn_exchange_arrive(scratch, unit);
+    if (!SHARED && p.split > 1 && tid == 0) arrived_before = gn_exchange_arrive(scratch, unit);
 
     // ---- token-major store: for each position of the slice one run of ch_per_group values
     const uint32_t rows = pvs * EPV;                         // positions in the slice
@@ -657,7 +679,7 @@ __global__ __launch_bounds__(kGnMaxThreads) void gn_tokens_kernel(
         }
         out[(size_t)r * row_stride + c] = w;
     }
-    if (p.split > 1 && tid == 0) gn_exchange_close(scratch, p, unit, epoch, arrived_before);
+    if (!SHARED && p.split > 1 && tid == 0) gn_exchange_close(scratch, p, unit, epoch, arrived_before);
 }
 
 // Any shape: one workgroup per unit, three passes, element-wise scattered stores.
@@ -1032,11 +1054,17 @@ template int gn_dispatch<__half>(const void *, const void *, void *, const float
 namespace {
 
 template <typename T, int K>
-void gn_tokens_launch(uint32_t blocks, uint32_t threads, size_t lds_bytes, hipStream_t stream,
+void gn_tokens_launch(bool shared, uint32_t blocks, uint32_t threads, size_t lds_bytes, hipStream_t stream,
                       const T *x, T *y, const float *gamma, const float *beta, const GnScratch &sc,
                       const GnTokParams &q) {
-    hipLaunchKernelGGL((gn_tokens_kernel<T, K>), dim3(blocks), dim3(threads), lds_bytes, stream, x, y,
-                       gamma, beta, sc, q);
+    if (K <= kGnSharedMaxK && shared) {
+        constexpr int KS = K <= kGnSharedMaxK ? K : 1;  // (no instances with several writers beyond that)
+        hipLaunchKernelGGL((gn_tokens_kernel<T, KS, true>), dim3(blocks), dim3(threads), lds_bytes, stream, x, y,
+                           gamma, beta, sc, q);
+    } else {
+        hipLaunchKernelGGL((gn_tokens_kernel<T, K, false>), dim3(blocks), dim3(threads), lds_bytes, stream, x, y,
+                           gamma, beta, sc, q);
+    }
 }
 
 }  // namespace
@@ -1084,19 +1112,49 @@ int gn_tokens_dispatch(const void *xv, void *yv, const float *gamma, const float
         split = s;
         if (s >= want) break;
     }
-    if (split == 0 || (split > 1 && units > kGnMaxUnits)) return generic();
+    // Several writers per whole unit instead of slices with an exchange (see gn_auto_writers): the
+    // parts cut the positions like slices do, must divide them, hold whole wavefronts' vectors
+    // and fit the LDS; the whole unit must fit the registers of one workgroup.
+    const int tune_writers = g_tuning.gn_writers.load(std::memory_order_relaxed);
+    uint32_t writers = 1;
+    const size_t vec_per_unit = cpg * hw_vec;
+    const char *xb = reinterpret_cast<const char *>(x), *yb = reinterpret_cast<const char *>(y);
+    const size_t bytes = units * unit_size * sizeof(T);
+    const bool apart = xb + bytes <= yb || yb + bytes <= xb;
+    if (apart && tune_split <= 1 && tune_writers != 1 && vec_per_unit <= (size_t)kGnMaxThreads * kGnSharedMaxK) {
+        uint32_t w = tune_writers > 1 ? (uint32_t)tune_writers : gn_auto_writers(sizeof(T), units, vec_per_unit);
+        // Here the limit is lower than for the channel-major store: the slices of a cut unit
+        // also keep the writers of an output line on one XCD, which the writers of a unit give
+        // up.  Measured, batch 2 fp16, several writers against slices: 1280 channels at 16 x 16
+        // 4.03 against 4.64 us, 640 at 32 x 32 5.79 against 6.11, 320 at 64 x 64 9.14 against
+        // 7.90; batch 4 (two writers): 4.72 against 5.13, 7.45 against 7.07.
+        if (tune_writers <= 1 && unit_size > (w >= 4 ? 20480u : 10240u)) w = 1;
+        for (; w > 1; w /= 2) {
+            if (hw_vec % w != 0) continue;
+            const size_t part_len = cpg * (hw_vec / w);
+            const size_t lds = cpg * (hw / w + 16 / sizeof(T)) * sizeof(T);
+            if (part_len % kWave == 0 && lds <= kMaxLds) break;
+        }
+        writers = w < 1 ? 1 : w;
+        if (writers > 1 &&
+            plan_slice((uint32_t)vec_per_unit, 1, 0, kGnSharedMaxK, true, units * writers, sizeof(T)).k == 0)
+            writers = 1;  // (the whole unit does not fit one workgroup's registers: slices as below)
+    }
+    const bool shared = writers > 1;
+    if (!shared && (split == 0 || (split > 1 && units > kGnMaxUnits))) return generic();
+    if (shared) split = 1;
 
     GnTokParams q;
-    const size_t pvs = hw_vec / split;
+    const size_t pvs = hw_vec / (shared ? writers : split);  // position vectors of a part / slice
     const size_t nvec = cpg * pvs;
-    q.base.vec_per_unit = (uint32_t)(nvec * split);
+    q.base.vec_per_unit = (uint32_t)vec_per_unit;
     q.base.vec_per_slice = (uint32_t)nvec;
     q.base.split = split;
     q.base.split_shift = (uint32_t)__builtin_ctz(split);
-    q.base.writers = 1;
-    q.base.writers_shift = 0;
-    q.base.part_vecs = 0;
-    q.base.same_xcd = 0;
+    q.base.writers = writers;
+    q.base.writers_shift = (uint32_t)__builtin_ctz(writers);
+    q.base.part_vecs = (uint32_t)nvec;
+    q.base.same_xcd = (shared && units % 8 == 0) ? 1u : 0u;
     q.base.groups = (uint32_t)groups;
     q.base.ch_per_group = (uint32_t)cpg;
     q.base.hw_vec = make_fast_div((uint32_t)hw_vec);
@@ -1109,26 +1167,30 @@ int gn_tokens_dispatch(const void *xv, void *yv, const float *gamma, const float
     q.channels = (uint32_t)channels;
     q.pitch = (uint32_t)(pvs * EPV + 16 / sizeof(T));
     q.combos = make_fast_div((uint32_t)(batch * split));
+    q.part_len = make_fast_div((uint32_t)nvec);
     const size_t lds_bytes = cpg * q.pitch * sizeof(T);
-    const GnPlan pl = plan_slice((uint32_t)nvec, split, 0, kMaxK, false);
+    // a workgroup holds its slice, or with several writers the whole unit
+    const GnPlan pl = shared ? plan_slice((uint32_t)vec_per_unit, 1, 0, kGnSharedMaxK, true, units * writers, sizeof(T))
+                             : plan_slice((uint32_t)nvec, split, 0, kMaxK, false);
     if (pl.k == 0) return generic();
     GnScratch sc{nullptr, nullptr, nullptr, nullptr, nullptr, 0};
-    if (split > 1) {
+    if (!shared && split > 1) {
         const hipError_t err = get_scratch(stream, &sc);
         if (err != hipSuccess) return (int)err;
     }
-    const uint32_t blocks = (uint32_t)(units * split);
+    const uint32_t blocks = (uint32_t)(units * (shared ? writers : split));
+    const uint32_t threads = pl.threads;
     switch (pl.k) {
-        case 1: gn_tokens_launch<T, 1>(blocks, pl.threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
-        case 2: gn_tokens_launch<T, 2>(blocks, pl.threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
-        case 3: gn_tokens_launch<T, 3>(blocks, pl.threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
-        case 4: gn_tokens_launch<T, 4>(blocks, pl.threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
-        case 5: gn_tokens_launch<T, 5>(blocks, pl.threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
-        case 6: gn_tokens_launch<T, 6>(blocks, pl.threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
-        case 8: gn_tokens_launch<T, 8>(blocks, pl.threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
-        case 10: gn_tokens_launch<T, 10>(blocks, pl.threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
-        case 12: gn_tokens_launch<T, 12>(blocks, pl.threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
-        default: gn_tokens_launch<T, 16>(blocks, pl.threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
+        case 1: gn_tokens_launch<T, 1>(shared, blocks, threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
+        case 2: gn_tokens_launch<T, 2>(shared, blocks, threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
+        case 3: gn_tokens_launch<T, 3>(shared, blocks, threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
+        case 4: gn_tokens_launch<T, 4>(shared, blocks, threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
+        case 5: gn_tokens_launch<T, 5>(shared, blocks, threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
+        case 6: gn_tokens_launch<T, 6>(shared, blocks, threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
+        case 8: gn_tokens_launch<T, 8>(shared, blocks, threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
+        case 10: gn_tokens_launch<T, 10>(shared, blocks, threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
+        case 12: gn_tokens_launch<T, 12>(shared, blocks, threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
+        default: gn_tokens_launch<T, 16>(shared, blocks, threads, lds_bytes, stream, x, y, gamma, beta, sc, q); break;
     }
     return launch_status();
 }

@@ -117,9 +117,12 @@ def test_add_layernorm_equals_two_launches(msd, orc, cuda, rows, dim, half):
                                                 ((1, 96, 24, 24), 32, 0), ((3, 64, 5, 7), 8, 0),
                                                 ((1, 33, 4, 4), 33, 0), ((1, 8, 128, 128), 1, 0),
                                                 ((8, 320, 32, 32), 32, 0), ((4, 640, 32, 32), 32, 0)])
-def test_groupnorm_tokens_equals_norm_then_permute(msd, orc, cuda, shape, groups, split, half):
+@pytest.mark.parametrize("writers", [0, 1, 4, 16], ids=["writers-auto", "one-writer", "4-writers", "16-writers"])
+def test_groupnorm_tokens_equals_norm_then_permute(msd, orc, cuda, shape, groups, split, half, writers):
     """SpatialTransformer's GroupNorm(eps 1e-6, no SiLU) + permute (0, 2, 1) in one launch
-    (M/nn/SpatialTransformer.cpp:127-139)."""
+    (M/nn/SpatialTransformer.cpp:127-139): slices of positions with an exchange, or (writers != 1,
+    where the shape allows it) several workgroups that each reduce the whole unit and store the
+    tokens of one range of positions."""
     import torch
     lib = msd.load_library()
     batch, channels = shape[0], shape[1]
@@ -130,9 +133,11 @@ def test_groupnorm_tokens_equals_norm_then_permute(msd, orc, cuda, shape, groups
     xd, gd, bd = _dev(xin, cuda, half), _dev(g, cuda), _dev(b, cuda)
     try:
         lib.msd_set_tuning(msd.TUNE_GN_SPLIT, split)
+        assert lib.msd_set_tuning(msd.TUNE_GN_WRITERS, writers) == 0
         fused = msd.groupnorm_tokens(xd, gd, bd, groups, 1e-6)
     finally:
         lib.msd_set_tuning(msd.TUNE_GN_SPLIT, 0)
+        lib.msd_set_tuning(msd.TUNE_GN_WRITERS, 0)
     two = msd.groupnorm(xd, gd, bd, groups, 1e-6, False).view(batch, channels, hw).permute(0, 2, 1).contiguous()
     assert fused.shape == (batch, hw, channels)
     # the slices cut positions instead of channel ranges, so the statistics are summed in another
