@@ -4,7 +4,8 @@ correct rounding of a 1e-5-accurate value, half an fp16 ulp plus 1e-5 relative a
 unrounded oracle, and 2e-3 below magnitude 4; adds, permute and the DDIM update bit-exact).
 The draws are seeded, so a failure names a reproducible case.  Shapes cover what the
 fixed-shape tests do not: odd lengths, tiny and huge groups, batches up to 40 (launches of
-many units), forced GroupNorm launch plans, rows that do not vectorise.
+many units), forced GroupNorm launch plans (workgroup size, slices, writers per unit), rows that
+do not vectorise.
 """
 
 import numpy as np
@@ -56,11 +57,13 @@ def gn_case():
     lib = msd.load_library()
     lib.msd_set_tuning(msd.TUNE_GN_THREADS, int(rng.choice([0, 0, 0, 64, 256, 320, 512, 640, 1024])))
     lib.msd_set_tuning(msd.TUNE_GN_SPLIT, int(rng.choice([0, 0, 0, 2, 4, 16])))
+    lib.msd_set_tuning(msd.TUNE_GN_WRITERS, int(rng.choice([0, 0, 1, 2, 4, 8, 16])))  # several workgroups per whole unit
     try:
         return _gn_case(groups, cpg, C, batch, hw, half, silu)
     finally:
         lib.msd_set_tuning(msd.TUNE_GN_THREADS, 0)
         lib.msd_set_tuning(msd.TUNE_GN_SPLIT, 0)
+        lib.msd_set_tuning(msd.TUNE_GN_WRITERS, 0)
 
 
 def _gn_case(groups, cpg, C, batch, hw, half, silu):
