@@ -17,6 +17,11 @@
 //   4. y = fma(x - mean, rstd * gamma[c], beta[c]) (the mean folded into the offset when it
 //      is small), optional SiLU, packed store.
 //
+// When the output lies apart from the input and the launch is small, whole units are instead
+// shared by several workgroups (SHARED): each loads and reduces the whole unit (steps 1 and 2,
+// the same bits in every one; the copies of the loads meet in the L2 of the XCD the writers are
+// placed on) and does step 4 for its own part of the unit.  No step 3, nothing waits.
+//
 // Workgroups of one unit have adjacent block ids, so a waiter's siblings are
 // normally dispatched together with it.  Nothing depends on that: a wait is
 // bounded (about a millisecond of polls), and a slice whose sibling has not
