@@ -383,7 +383,10 @@ def launch_floor_us(torch, msd, dev, stream):
 def gn_split_table(torch, msd, dev, stream):
     """GroupNorm+SiLU at the config-2 shapes with the launch plan forced: workgroups per
     (sample, group) in {1, 2, 4, 8} x workgroup size in {512, 1024}, next to the automatic
-    plan.  `auto_vs_best` > 1.03 would mean the plan in groupnorm.hip picks a slow variant."""
+    plan, all with one writer per unit (what a call in place gets: slices with an exchange).
+    `auto_vs_best` > 1.03 would mean the plan in groupnorm.hip picks a slow variant.  `writers`
+    is the automatic plan of a call whose output lies apart from its input (several workgroups
+    share each whole unit), which is how this table's buffers are laid out."""
     lib = msd.load_library()
     rows = []
     for c, side in [(320, 64), (640, 32), (1280, 16), (1280, 8), (960, 32), (1920, 16)]:
@@ -391,6 +394,10 @@ def gn_split_table(torch, msd, dev, stream):
             case = _kernel_case(torch, msd, dev, "groupnorm_silu", {"c": c, "hw": side * side}, dt, BATCH)
             times = {}
             try:
+                assert lib.msd_set_tuning(msd.TUNE_GN_WRITERS, 0) == 0
+                writers_us = round(_rotating_launch_us(torch, msd, stream, case["launch"], case["xs"], case["ys"],
+                                                       budget=1000), 3)
+                assert lib.msd_set_tuning(msd.TUNE_GN_WRITERS, 1) == 0
                 for split in (0, 1, 2, 4, 8):
                     for threads in ((0,) if split == 0 else (512, 1024)):
                         assert lib.msd_set_tuning(msd.TUNE_GN_SPLIT, split) == 0
@@ -401,9 +408,12 @@ def gn_split_table(torch, msd, dev, stream):
             finally:
                 lib.msd_set_tuning(msd.TUNE_GN_SPLIT, 0)
                 lib.msd_set_tuning(msd.TUNE_GN_THREADS, 0)
+                lib.msd_set_tuning(msd.TUNE_GN_WRITERS, 0)
             best = min(v for k, v in times.items() if k != "auto")
             rows.append({"shape": {"c": c, "hw": side * side, "batch": BATCH}, "dtype": "f16" if case["elt"] == 2 else "f32",
-                         "us": times, "best_forced_us": best, "auto_vs_best": round(times["auto"] / best, 3)})
+                         "us": times, "best_forced_us": best, "auto_vs_best": round(times["auto"] / best, 3),
+                         "writers_us": writers_us, "writers_plan": _gn_plan_text(msd, BATCH, c, side * side, case["elt"]),
+                         "writers_vs_auto": round(writers_us / times["auto"], 3)})
             del case
             torch.cuda.empty_cache()
     return rows
