@@ -891,6 +891,7 @@ GnDecision gn_decide(size_t elt, size_t batch, size_t channels, size_t hw, size_
     if (may_share && tune_split <= 1 && tune_writers != 1 && vec_per_unit <= (size_t)kGnMaxThreads * kGnSharedMaxK) {
         uint32_t writers = tune_writers > 1 ? (uint32_t)tune_writers : gn_auto_writers(elt, units, vec_per_unit);
         while (writers > 1 && vec_per_unit < (size_t)writers * kWave) writers /= 2;  // a part is at least a wavefront's vectors
+        if (units * writers > 0x7FFFFFFFull) writers = 1;                            // (the grid is units * writers blocks)
         if (writers > 1) {
             uint32_t force = 0;
             if (tune_threads >= kWave && tune_threads <= kGnMaxThreads && tune_threads % kWave == 0 &&
@@ -1140,7 +1141,7 @@ int gn_tokens_dispatch(const void *xv, void *yv, const float *gamma, const float
             const size_t lds = cpg * (hw / w + 16 / sizeof(T)) * sizeof(T);
             if (part_len % kWave == 0 && lds <= kMaxLds) break;
         }
-        writers = w < 1 ? 1 : w;
+        writers = (w < 1 || units * w > 0x7FFFFFFFull) ? 1 : w;  // (the grid is units * writers blocks)
         if (writers > 1 &&
             plan_slice((uint32_t)vec_per_unit, 1, 0, kGnSharedMaxK, true, units * writers, sizeof(T)).k == 0)
             writers = 1;  // (the whole unit does not fit one workgroup's registers: slices as below)
