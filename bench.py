@@ -726,7 +726,11 @@ def step_with_adds(torch, msd, dev, stream):
     those launches (time_embed_0 / SiLU / time_embed_2, M/UNetModel.cpp:1107-1120, and SiLU(emb)
     -> embed_linear in every ResBlock, M/nn/ResBlock.cpp:173-183, whose output is what the
     embedding add adds): every launch separate, against SiLU folded into the Linear kernels and
-    the 22 projections as ONE grouped launch ahead of the blocks."""
+    the 22 projections as ONE grouped launch ahead of the blocks.
+
+    A third pair adds the 16 SpatialTransformer norms (GroupNorm without SiLU, then the permute to
+    tokens, M/nn/SpatialTransformer.cpp:127-139) as two launches each, against the one launch of
+    msd_groupnorm_tokens."""
     import ctypes
     vp = ctypes.c_void_p
     lib = msd.load_library()
@@ -748,6 +752,7 @@ def step_with_adds(torch, msd, dev, stream):
 
     separate, fused = [], []  # lists of (fn, args)
     separate_emb, fused_emb = [], []  # the same with the embedding-row Linear layers
+    st_separate, st_fused = [], []    # the SpatialTransformer norms: GroupNorm + permute against one launch
     # embedding path: sinusoid [2, 320] -> h [2, 1280] -> emb [2, 1280] -> per ResBlock [2, Cout]
     couts = [c for _, c, _ in RESBLOCKS]
     temb_out = torch.empty((BATCH, 320), device=dev, dtype=torch.float16)
@@ -826,6 +831,18 @@ def step_with_adds(torch, msd, dev, stream):
             ga, be = gb(dim)
             xp, yp, gp, bp = vp(x.data_ptr()), vp(y.data_ptr()), vp(ga.data_ptr()), vp(be.data_ptr())
             if ln_count % 3 == 0:  # LayerNorm 1 of a block has no add in front
+                # the SpatialTransformer's own norm ahead of the block (M/nn/SpatialTransformer.cpp:127-139):
+                # GroupNorm(eps 1e-6, no SiLU) over [B, dim, tokens], then the permute to [B, tokens, dim]
+                sx = randn(BATCH, dim, rows // BATCH) * 2.0
+                sy, sz = torch.empty_like(sx), torch.empty_like(sx)
+                keep.extend([sy, sz])
+                sga, sbe = gb(dim)
+                sxp, syp, szp = vp(sx.data_ptr()), vp(sy.data_ptr()), vp(sz.data_ptr())
+                st_separate.append((lib.msd_groupnorm, (sxp, syp, vp(sga.data_ptr()), vp(sbe.data_ptr()), BATCH, dim,
+                                                        rows // BATCH, 32, 1e-6, 0, F16)))
+                st_separate.append((lib.msd_permute_0_2_1, (syp, szp, BATCH, dim, rows // BATCH, F16)))
+                st_fused.append((lib.msd_groupnorm_tokens, (sxp, szp, vp(sga.data_ptr()), vp(sbe.data_ptr()), BATCH, dim,
+                                                            rows // BATCH, 32, 1e-6, F16)))
                 call = (lib.msd_layernorm, (xp, yp, gp, bp, rows, dim, 1e-5, F16))
                 for lst in (separate, fused, separate_emb, fused_emb):
                     lst.append(call)
@@ -855,8 +872,9 @@ def step_with_adds(torch, msd, dev, stream):
         return run
 
     out = {}
+    separate_all, fused_all = separate_emb + st_separate, fused_emb + st_fused
     for name, calls in (("separate", separate), ("fused", fused), ("separate_emb", separate_emb),
-                        ("fused_emb", fused_emb)):
+                        ("fused_emb", fused_emb), ("separate_all", separate_all), ("fused_all", fused_all)):
         replay = capture(torch, msd, stream, runner(calls))
         with torch.cuda.stream(stream):
             for _ in range(5):
@@ -868,7 +886,11 @@ def step_with_adds(torch, msd, dev, stream):
             "with_embedding_linears": {
                 "launches_separate": len(separate_emb), "launches_fused_grouped": len(fused_emb),
                 "ms_separate": round(out["separate_emb"], 4), "ms_fused_grouped": round(out["fused_emb"], 4),
-                "speedup": round(out["separate_emb"] / out["fused_emb"], 3)}}
+                "speedup": round(out["separate_emb"] / out["fused_emb"], 3)},
+            "with_spatial_transformer_norms_too": {
+                "launches_separate": len(separate_all), "launches_fused": len(fused_all),
+                "ms_separate": round(out["separate_all"], 4), "ms_fused": round(out["fused_all"], 4),
+                "speedup": round(out["separate_all"] / out["fused_all"], 3)}}
 
 
 def cpu_baseline(total_bytes, budget_s=24.0):
