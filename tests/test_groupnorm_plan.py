@@ -64,12 +64,12 @@ def test_plans_of_the_unet_shapes_at_batch_2_and_32():
     # output apart from the input: up to 256 workgroups share whole units of up to 5120 vectors
     # (10240 of 4-byte elements with up to four writers); larger units and batches plan as above
     apart = {
-        (2, 320, 4096, f16): (1, 1024, 5, 4), (2, 640, 1024, f16): (1, 512, 5, 4), (2, 1280, 256, f16): (1, 512, 3, 4),
-        (2, 1280, 64, f16): (1, 320, 1, 4), (2, 960, 1024, f16): (1, 1024, 4, 4), (2, 1920, 256, f16): (1, 960, 2, 4),
+        (2, 320, 4096, f16): (1, 1024, 5, 4), (2, 640, 1024, f16): (1, 640, 4, 4), (2, 1280, 256, f16): (1, 512, 3, 4),
+        (2, 1280, 64, f16): (1, 384, 1, 4), (2, 960, 1024, f16): (1, 1024, 4, 4), (2, 1920, 256, f16): (1, 512, 4, 4),
         (2, 1920, 1024, f16): (4, 960, 2, 1), (2, 640, 4096, f16): (4, 1024, 3, 1),
-        (1, 320, 4096, f16): (1, 1024, 5, 8), (1, 1280, 64, f16): (1, 320, 1, 4), (4, 640, 1024, f16): (1, 512, 5, 2),
+        (1, 320, 4096, f16): (1, 1024, 5, 8), (1, 1280, 64, f16): (1, 384, 1, 4), (4, 640, 1024, f16): (1, 640, 4, 2),
         (1, 320, 4096, f32): (4, 640, 4, 1), (1, 640, 1024, f32): (1, 1024, 5, 8), (2, 320, 4096, f32): (1, 1024, 10, 4),
-        (2, 960, 1024, f32): (1, 1024, 8, 4), (2, 960, 4096, f32): (8, 960, 4, 1),
+        (2, 960, 1024, f32): (1, 1024, 8, 4), (2, 960, 4096, f32): (8, 960, 4, 1), (2, 1280, 256, f32): (1, 640, 4, 4),
         (8, 320, 4096, f16): (1, 1024, 5, 1), (32, 320, 4096, f16): (1, 256, 20, 1),
     }
     for (batch, channels, hw, code), want in apart.items():
