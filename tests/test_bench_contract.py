@@ -1,6 +1,6 @@
 """bench.py's workload definition and command line, checked without a GPU: the step is BASELINE
 config 5 (one timestep embedding, 23 SiLU on the embedding, 45 GroupNorm+SiLU, 48 LayerNorm,
-16 GEGLU at the SD UNet shapes, batch 2, fp16) with the algorithmic bytes of the survey's table,
+16 GEGLU at the SD UNet shapes, batch 2, fp16) with the algorithmic bytes that follow from those shapes,
 in the reference's order (M/nn/ResBlock.cpp:125-232, M/nn/BasicTransformerBlock.cpp:116-164,
 M/UNetModel.cpp:1796-1810), and a run on more than one GPU is refused."""
 import os

@@ -10,8 +10,8 @@ fp16 storage : the oracle runs in fp32 on inputs already rounded to fp16; its UN
                rejects truncation, a wrong rounding mode and a value that is a whole ulp off.
 
 Every fp16 check also records, per label, the worst error and how many elements exceed a bare
-2e-3 (all of them sit above |ref32| = 4 if the assertion held); the GPU run writes the table
-to gpurun_out/parity_fp16.json.
+2e-3 (all of them sit above |ref32| = 4 if the assertion held); at the end of a GPU run
+conftest.py writes the table as parity_fp16.json into the run's output folder.
 """
 import numpy as np
 
