@@ -221,7 +221,10 @@ def test_softmax_attention_shapes(msd, orc, cuda, rows, cols, stable, half):
 
 @pytest.mark.parametrize("rows,cols", [(1, 1), (3, 4), (5, 8), (9, 40), (7, 300), (4, 600), (6, 1000),
                                        (3, 2048), (5, 8192), (2, 10000), (33, 129), (2, 513),
-                                       (200, 100), (128, 9), (64, 128), (191, 127), (70, 8)])
+                                       (200, 100), (128, 9), (64, 128), (191, 127), (70, 8),
+                                       # rows of 3 ... 66 vectors: every team size of the register kernel,
+                                       # row counts that leave part of the last wavefront without a row
+                                       (67, 24), (35, 32), (50, 96), (45, 200), (21, 136), (19, 264)])
 def test_softmax_edge_shapes(msd, orc, cuda, rows, cols):
     for half in (False, True):
         for stable in (0, 1):
