@@ -254,19 +254,28 @@ __global__ __launch_bounds__(kLnThreads) void ln_generic_kernel(
 template <typename T, int NW, int VPL, int TL>
 void ln_launch(const T *x, const T *res, T *sum, T *y, const float *gamma, const float *beta,
                uint32_t rows, float eps, float inv_dim, hipStream_t stream) {
-    // one wavefront per workgroup is 2 - 8 % faster while the launch is small (measured below
-    // about 1000 wavefronts); large launches dispatch sooner as 4-wavefront workgroups
+    // Up to one wavefront per SIMD of the chip (1024) the launch is bound by its own latency chain:
+    // one wavefront per workgroup (1 - 5 % faster than four), gamma / beta requested together with
+    // the row.  From two wavefronts per SIMD on throughput counts: gamma / beta through LDS (fewer
+    // load instructions and registers per wavefront), four wavefronts per workgroup, two for
+    // launches of 4096 up to 10240 wavefronts (3 - 19 % faster there, 1 - 7 % slower at 3072 and
+    // from 10240 on).  Measured, us per launch, with the row / LDS x 64, 128, 256 lanes:
+    //   fp16 8192 x 320 (1024 wavefronts)   3.54 3.71 3.59 / 3.57 3.88 3.57
+    //   fp16 16384 x 320 (2048)             5.12 5.19 5.22 / 4.94 4.78 4.94
+    //   fp32 8192 x 320 (2048)              5.28 5.29 5.17 / 4.90 4.71 4.99
+    //   fp16 8192 x 1024 (8192)             8.19 8.01 8.17 / 9.32 7.09 7.96
+    //   fp16 16384 x 768 (8192)             11.8 12.1 12.2 / 12.1 9.54 10.7
+    //   fp16 8192 x 1280 (4096)             10.4 10.6 10.4 / 8.19 7.95 7.95
+    //   fp16 32768 x 1024 (32768)           24.5 24.5 24.5 / 31.7 25.0 24.1
     const uint32_t wavefronts = (rows + (kWave / TL) - 1) / (kWave / TL);
+    const bool early = wavefronts < 2048;
     const int tune_threads = g_tuning.ln_threads.load(std::memory_order_relaxed);
     const uint32_t threads = tune_threads ? (uint32_t)tune_threads
-                                                 : (wavefronts >= 1024 ? 256u : (uint32_t)kLnThreads);
+                             : early      ? (wavefronts <= 1024 ? (uint32_t)kLnThreads : 256u)
+                                          : (wavefronts >= 4096 && wavefronts < 10240 ? 128u : 256u);
     const uint32_t rows_per_block = (kWave / TL) * (threads / kWave);
     const uint32_t blocks = (rows + rows_per_block - 1) / rows_per_block;
-    // a launch of up to two wavefronts per SIMD of the chip is bound by its own latency chain:
-    // gamma / beta come with the row; beyond that by throughput: fewer registers per wavefront
-    // (measured: 8192 x 1280 fp16, 4096 wavefronts: 8.5 us late against 10.6 us early;
-    // 8192 x 320, 1024 wavefronts: 3.6 us early against 3.9 us late)
-    if (wavefronts <= 2048)
+    if (early)
         hipLaunchKernelGGL((ln_team_kernel<T, NW, VPL, TL, true>), dim3(blocks), dim3(threads), 0, stream, x,
                            res, sum, y, gamma, beta, rows, eps, inv_dim);
     else
