@@ -519,7 +519,8 @@ def fusion_table(torch, msd, dev, stream):
 def neighbour_table(torch, msd, dev, stream):
     """The kernels either side of the path: attention row softmax (fp16, in place) next to a
     plain copy of the same bytes, the Linear layers on the time-embedding rows with the SiLU
-    folded in or launched separately, and the DDIM latent update (graph-replayed)."""
+    folded in or launched separately, the stand-alone permute next to a copy, and the DDIM latent
+    update (graph-replayed)."""
     import ctypes
     vp = ctypes.c_void_p
     lib = msd.load_library()
@@ -631,6 +632,26 @@ def neighbour_table(torch, msd, dev, stream):
                      "bytes": nbytes, "us": round(us_grp, 2), "GBps": round(nbytes / us_grp / 1e3, 1),
                      "us_22_launches": round(us_sep, 2), "speedup": round(us_sep / us_grp, 2)})
         del ws, tables
+        torch.cuda.empty_cache()
+
+    # tokens -> NCHW behind a SpatialTransformer (the permute that stays a launch of its own), next
+    # to a plain copy of the same bytes
+    for tokens, dim in [(4096, 320), (1024, 640), (256, 1280)]:
+        count = BATCH * tokens * dim
+        nbytes = 2 * count * 2
+        copies = max(4, min(32, int(300e6 // nbytes)))
+        xs = [torch.randn(count, device=dev).half() for _ in range(copies)]
+        ys = [torch.empty(count, device=dev, dtype=torch.float16) for _ in range(copies)]
+        us = _rotating_launch_us(torch, msd, stream, lambda x, y, s_: lib.msd_permute_0_2_1(
+            vp(x.data_ptr()), vp(y.data_ptr()), BATCH, tokens, dim, F16, s_), xs, ys, budget=600)
+        cus = _rotating_launch_us(torch, msd, stream, lambda x, y, s_: lib.msd_copy(
+            vp(x.data_ptr()), vp(y.data_ptr()), count * 2, s_), xs, ys, budget=600)
+        gbs = nbytes / us / 1e3
+        rows.append({"kernel": "permute_0_2_1", "shape": {"i": BATCH, "j": tokens, "k": dim}, "dtype": "f16",
+                     "bytes": nbytes, "us": round(us, 2), "GBps": round(gbs, 1),
+                     "pct_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 1), "copy_us": round(cus, 2),
+                     "pct_of_copy_rate": round(100 * cus / us, 1)})
+        del xs, ys
         torch.cuda.empty_cache()
 
     # DDIM update of the latent, batch 2 x [4, 64, 64] float32, in place

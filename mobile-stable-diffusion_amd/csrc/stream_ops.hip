@@ -182,6 +182,79 @@ __global__ __launch_bounds__(256) void permute_021_kernel(const T *__restrict__ 
     }
 }
 
+// The same permute with 16-byte accesses on both sides and an LDS tile of 32-bit words that is
+// written transposed: tile[k][w] holds word w of output row k (one 4-byte element, or the 2-byte
+// elements of input rows 2w and 2w + 1 at column k, paired in registers after the load), with an
+// odd pitch, so that the 32-bit writes of a wavefront (one column per lane) and its 32-bit reads
+// (four adjacent words per lane) each fall on all banks.  ES = bytes per element; a workgroup moves
+// 64 x 64 elements; jsize and ksize are multiples of 16 / ES (host), so a 16-byte piece is all
+// inside the tensor or all outside.
+template <int ES>
+__global__ __launch_bounds__(256) void permute_021_words_kernel(const void *__restrict__ srcv,
+                                                                void *__restrict__ dstv, uint32_t jsize,
+                                                                uint32_t ksize) {
+    constexpr uint32_t EPV = 16 / ES;               // elements per 16-byte piece
+    constexpr uint32_t kWords = kTile * ES / 4;     // 32-bit words per output row of the tile
+    constexpr uint32_t kPitch = kWords + 1;
+    __shared__ uint32_t tile[kTile * kPitch];
+    const uint32_t k0 = blockIdx.x * kTile, j0 = blockIdx.y * kTile, i = blockIdx.z;
+    const size_t plane = (size_t)i * jsize * ksize;  // in elements
+    const char *in = static_cast<const char *>(srcv) + plane * ES;
+    char *out = static_cast<char *>(dstv) + plane * ES;
+    const uint32_t t = threadIdx.x;
+    if (ES == 4) {
+        // a lane loads elements k .. k+3 of one input row; 16 lanes cover the tile's 64 columns
+        // (all four loads leave before the first LDS write: a piece outside the tensor re-reads
+        // the plane's first piece instead of sitting behind a branch)
+        const uint32_t kq = (t & 15) * 4, jr = t >> 4, k = k0 + kq;
+        u32x4 v[4];
+#pragma unroll
+        for (int pass = 0; pass < 4; pass++) {
+            const uint32_t j = j0 + jr + pass * 16;
+            const size_t at = (j < jsize && k < ksize) ? ((size_t)j * ksize + k) * 4 : 0;
+            v[pass] = load_stream(reinterpret_cast<const u32x4 *>(in + at));
+        }
+#pragma unroll
+        for (int pass = 0; pass < 4; pass++) {
+            const uint32_t jl = jr + pass * 16;
+            if (j0 + jl < jsize && k < ksize) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) tile[(kq + e) * kPitch + jl] = v[pass][e];
+            }
+        }
+    } else {
+        // a lane loads elements k .. k+7 of input rows j and j+1 and pairs them by column
+        const uint32_t kq = (t & 7) * 8, jw = t >> 3;  // jw: word of the output rows, 0 .. 31
+        const uint32_t j = j0 + 2 * jw, k = k0 + kq;
+        if (j < jsize && k < ksize) {  // (jsize is even: row j + 1 exists)
+            const u32x4 a = load_stream(reinterpret_cast<const u32x4 *>(in + ((size_t)j * ksize + k) * 2));
+            const u32x4 b = load_stream(reinterpret_cast<const u32x4 *>(in + ((size_t)(j + 1) * ksize + k) * 2));
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                tile[(kq + 2 * w) * kPitch + jw] = (a[w] & 0xffffu) | (b[w] << 16);
+                tile[(kq + 2 * w + 1) * kPitch + jw] = (a[w] >> 16) | (b[w] & 0xffff0000u);
+            }
+        }
+    }
+    __syncthreads();
+    // a lane stores one 16-byte piece (four words) of an output row
+    constexpr uint32_t kPieces = kWords / 4;         // pieces per output row of the tile: 16 or 8
+    constexpr uint32_t kRowsPerPass = 256 / kPieces;  // 16 or 32
+    const uint32_t wq = (t % kPieces) * 4, kr = t / kPieces;
+    constexpr uint32_t kPasses = kTile / kRowsPerPass;
+    u32x4 w[kPasses];
+#pragma unroll
+    for (uint32_t pass = 0; pass < kPasses; pass++) {  // (words of pieces outside the tensor are never stored)
+#pragma unroll
+        for (int e = 0; e < 4; e++) w[pass][e] = tile[(kr + pass * kRowsPerPass) * kPitch + wq + e];
+    }
+#pragma unroll
+    for (uint32_t pass = 0; pass < kPasses; pass++) {
+        const uint32_t k = k0 + kr + pass * kRowsPerPass, j = j0 + wq * (4 / ES);
+        if (k < ksize && j < jsize) store_stream(reinterpret_cast<u32x4 *>(out + ((size_t)k * jsize + j) * ES), w[pass]);
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(kStreamThreads) void permute_021_generic_kernel(
     const T *__restrict__ src, T *__restrict__ dst, size_t isize, size_t jsize, size_t ksize) {
@@ -327,7 +400,13 @@ int permute_021_dispatch(const void *srcv, void *dstv, size_t isize, size_t jsiz
     const bool tiled = jsize % 4 == 0 && ksize % 4 == 0 && reinterpret_cast<uintptr_t>(src) % piece == 0 &&
                        reinterpret_cast<uintptr_t>(dst) % piece == 0 && isize <= 65535 &&
                        (jsize + kTile - 1) / kTile <= 65535 && ksize < 0x7FFFFFFFull && jsize < 0x7FFFFFFFull;
-    if (tiled) {
+    const size_t epv = 16 / sizeof(T);
+    const bool words = tiled && jsize % epv == 0 && ksize % epv == 0 && aligned16(src) && aligned16(dst);
+    const dim3 tiles((uint32_t)((ksize + kTile - 1) / kTile), (uint32_t)((jsize + kTile - 1) / kTile), (uint32_t)isize);
+    if (words) {
+        hipLaunchKernelGGL((permute_021_words_kernel<(int)sizeof(T)>), tiles, dim3(256), 0, stream, srcv, dstv,
+                           (uint32_t)jsize, (uint32_t)ksize);
+    } else if (tiled) {
         hipLaunchKernelGGL((permute_021_kernel<T>),
                            dim3((uint32_t)((ksize + kTile - 1) / kTile), (uint32_t)((jsize + kTile - 1) / kTile),
                                 (uint32_t)isize),

@@ -161,7 +161,9 @@ def test_groupnorm_tokens_equals_norm_then_permute(msd, orc, cuda, shape, groups
 
 @pytest.mark.parametrize("half", [False, True], ids=["f32", "f16"])
 @pytest.mark.parametrize("shape", [(2, 320, 4096), (2, 4096, 320), (1, 1280, 64), (3, 100, 36), (2, 7, 5),
-                                   (1, 64, 64), (5, 68, 132), (1, 1, 8)])
+                                   (1, 64, 64), (5, 68, 132), (1, 1, 8),
+                                   # 16-byte pieces on both sides with ragged tiles, one tile, thin planes
+                                   (3, 72, 200), (2, 8, 8), (1, 136, 64), (2, 16, 1000), (4, 264, 24)])
 def test_permute_0_2_1(msd, orc, cuda, shape, half):
     import torch
     x = orc.normal(shape, seed=sum(shape))
