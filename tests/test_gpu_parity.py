@@ -394,6 +394,31 @@ def test_layernorm_dims_and_ragged_rows(msd, orc, cuda, rows, dim, half):
         assert_close_f32(got, ref, what="ln dims f32")
 
 
+@pytest.mark.parametrize("half", [False, True], ids=["f32", "f16"])
+@pytest.mark.parametrize("rows,dim", [(2049, 1024), (5001, 1024), (10241, 768), (16387, 320), (9001, 640),
+                                      (4097, 1280)])
+def test_layernorm_mid_size_launches_with_ragged_ends(msd, orc, cuda, rows, dim, half):
+    # launches of 2048 ... 10240 wavefronts: gamma / beta through LDS in workgroups of two or
+    # four wavefronts, the last workgroup only partly filled with rows; alone and with the
+    # residual added first
+    x = orc.normal((rows, dim), seed=rows + dim, sigma=1.5, mean=0.5)
+    r = orc.normal((rows, dim), seed=rows + dim + 1)
+    if half:
+        x, r = orc.round_to_half(x), orc.round_to_half(r)
+    g, b = _affine(orc, dim, dim)
+    gd, bd = _to_dev(g, cuda), _to_dev(b, cuda)
+    check = (lambda got, ref, what: assert_close_f16(got, ref.astype(np.float32), what)) if half else \
+            (lambda got, ref, what: assert_close_f32(got, ref, what=what))
+    got = msd.layernorm(_to_dev(x, cuda, half), gd, bd).float().cpu().numpy()
+    check(got, orc.layernorm64(x, g, b, 1e-5), "ln mid-size")
+    s = x + r
+    if half:
+        s = orc.round_to_half(s)
+    sm, got = msd.add_layernorm(_to_dev(x, cuda, half), _to_dev(r, cuda, half), gd, bd, 1e-5)
+    assert np.array_equal(sm.float().cpu().numpy(), s.astype(np.float32))
+    check(got.float().cpu().numpy(), orc.layernorm64(s.astype(np.float32), g, b, 1e-5), "add + ln mid-size")
+
+
 @pytest.mark.parametrize("chunk,threads", [(8, 0), (16, 0), (8, 64), (16, 512), (0, 128)])
 def test_layernorm_forced_chunk_width(msd, orc, cuda, chunk, threads):
     lib = msd.load_library()
