@@ -6,6 +6,10 @@
  * default stream).  Calls are asynchronous on that stream.  Return value: 0 on
  * success, otherwise a hipError_t value (1 = hipErrorInvalidValue is also used
  * for rejected shapes / null pointers / unknown dtype).  No call throws.
+ * Where an output may take the place of an input ("may alias") it must be exactly
+ * that input or lie apart from it, and where it must not overlap an input no byte
+ * may be shared: any other overlap is refused with hipErrorInvalidValue before
+ * anything is launched.
  *
  * Each entry point names the reference interface it replaces (paths relative to
  * app/src/main of 9Hyeonwoo/mobile-stable-diffusion; K/ = assets/kernel/,

@@ -233,12 +233,29 @@ int msd_set_tuning(int knob, int value) {
     }
 }
 
+// Byte ranges [a, a + abytes) and [b, b + bbytes) share at least one byte.
+static bool ranges_overlap(const void *a, size_t abytes, const void *b, size_t bbytes) {
+    const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
+    return abytes != 0 && bbytes != 0 && a0 < b0 + bbytes && b0 < a0 + abytes;
+}
+// An output that may take the place of its input must be exactly that input or lie apart from
+// it: a shifted overlap would let one workgroup store into what another still has to load.
+static bool shifted_overlap(const void *in, const void *out, size_t bytes) {
+    return in != out && ranges_overlap(in, bytes, out, bytes);
+}
+static size_t elt_bytes(int dtype) { return dtype == MSD_DTYPE_F32 ? 4 : 2; }
+
 static int groupnorm_entry(const void *x, const void *chunk, void *y, const float *gamma,
                            const float *beta, size_t batch, size_t channels, size_t hw, size_t groups,
                            float eps, int fuse_silu, int dtype, const GnScratch *fixed, void *stream) {
     if (groups == 0 || channels == 0 || channels % groups != 0) return MSD_ERR_INVALID_VALUE;
     if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
     if (batch * hw != 0 && (!x || !y || !gamma || !beta)) return MSD_ERR_INVALID_VALUE;
+    size_t count;
+    if (__builtin_mul_overflow(batch, channels, &count) || __builtin_mul_overflow(count, hw, &count) ||
+        count > (SIZE_MAX >> 3))
+        return MSD_ERR_INVALID_VALUE;
+    if (shifted_overlap(x, y, count * elt_bytes(dtype))) return MSD_ERR_INVALID_VALUE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == MSD_DTYPE_F32)
         return gn_dispatch<float>(x, chunk, y, gamma, beta, batch, channels, hw, groups, eps,
@@ -298,7 +315,12 @@ int msd_groupnorm_tokens(const void *x, void *y, const float *gamma, const float
                          void *stream) {
     if (groups == 0 || channels == 0 || channels % groups != 0) return MSD_ERR_INVALID_VALUE;
     if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
-    if (batch * hw != 0 && (!x || !y || !gamma || !beta || x == y)) return MSD_ERR_INVALID_VALUE;
+    if (batch * hw != 0 && (!x || !y || !gamma || !beta)) return MSD_ERR_INVALID_VALUE;
+    size_t count;
+    if (__builtin_mul_overflow(batch, channels, &count) || __builtin_mul_overflow(count, hw, &count) ||
+        count > (SIZE_MAX >> 3))
+        return MSD_ERR_INVALID_VALUE;
+    if (ranges_overlap(x, count * elt_bytes(dtype), y, count * elt_bytes(dtype))) return MSD_ERR_INVALID_VALUE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == MSD_DTYPE_F32)
         return gn_tokens_dispatch<float>(x, y, gamma, beta, batch, channels, hw, groups, eps, s);
@@ -310,6 +332,13 @@ static int layernorm_entry(const void *x, const void *res, void *sum, void *y, c
                            void *stream) {
     if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
     if (rows * dim != 0 && (!x || !y || !gamma || !beta)) return MSD_ERR_INVALID_VALUE;
+    size_t count;
+    if (__builtin_mul_overflow(rows, dim, &count) || count > (SIZE_MAX >> 3)) return MSD_ERR_INVALID_VALUE;
+    const size_t bytes = count * elt_bytes(dtype);
+    if (shifted_overlap(x, y, bytes)) return MSD_ERR_INVALID_VALUE;
+    if (res != nullptr && (shifted_overlap(x, sum, bytes) || shifted_overlap(res, sum, bytes) ||
+                           ranges_overlap(sum, bytes, y, bytes) || shifted_overlap(res, y, bytes)))
+        return MSD_ERR_INVALID_VALUE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == MSD_DTYPE_F32)
         return ln_dispatch<float>(x, res, sum, y, gamma, beta, rows, dim, eps, s);
@@ -331,6 +360,9 @@ int msd_add_layernorm(const void *a, const void *b, void *sum, void *y, const fl
 int msd_elemwise_add(const void *a, const void *b, void *c, size_t n, int dtype, void *stream) {
     if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
     if (n != 0 && (!a || !b || !c)) return MSD_ERR_INVALID_VALUE;
+    if (n > (SIZE_MAX >> 3)) return MSD_ERR_INVALID_VALUE;
+    if (shifted_overlap(a, c, n * elt_bytes(dtype)) || shifted_overlap(b, c, n * elt_bytes(dtype)))
+        return MSD_ERR_INVALID_VALUE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == MSD_DTYPE_F32) return add_dispatch<float>(a, b, c, n, 0, s);
     return add_dispatch<__half>(a, b, c, n, 0, s);
@@ -341,6 +373,10 @@ int msd_chunkwise_add(const void *a, const void *chunk, void *c, size_t n, size_
     if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
     if (chunk_size == 0) return MSD_ERR_INVALID_VALUE;
     if (n != 0 && (!a || !chunk || !c)) return MSD_ERR_INVALID_VALUE;
+    if (n > (SIZE_MAX >> 3)) return MSD_ERR_INVALID_VALUE;
+    if (shifted_overlap(a, c, n * elt_bytes(dtype)) ||
+        ranges_overlap(chunk, (n / chunk_size) * elt_bytes(dtype), c, n * elt_bytes(dtype)))
+        return MSD_ERR_INVALID_VALUE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == MSD_DTYPE_F32) return add_dispatch<float>(a, chunk, c, n, chunk_size, s);
     return add_dispatch<__half>(a, chunk, c, n, chunk_size, s);
@@ -363,6 +399,7 @@ int msd_geglu(const void *proj, void *out, size_t rows, size_t inner, int dtype,
 static int act_entry(Act op, const void *x, void *y, size_t n, int dtype, void *stream) {
     if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
     if (n != 0 && (!x || !y)) return MSD_ERR_INVALID_VALUE;
+    if (n > (SIZE_MAX >> 3) || shifted_overlap(x, y, n * elt_bytes(dtype))) return MSD_ERR_INVALID_VALUE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == MSD_DTYPE_F32) return act_dispatch<float>(op, x, y, n, s);
     return act_dispatch<__half>(op, x, y, n, s);
@@ -381,7 +418,12 @@ int msd_quick_gelu(const void *x, void *y, size_t n, int dtype, void *stream) {
 int msd_permute_0_2_1(const void *src, void *dst, size_t isize, size_t jsize, size_t ksize, int dtype,
                       void *stream) {
     if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
-    if (isize * jsize * ksize != 0 && (!src || !dst || src == dst)) return MSD_ERR_INVALID_VALUE;
+    if (isize * jsize * ksize != 0 && (!src || !dst)) return MSD_ERR_INVALID_VALUE;
+    size_t count;
+    if (__builtin_mul_overflow(isize, jsize, &count) || __builtin_mul_overflow(count, ksize, &count) ||
+        count > (SIZE_MAX >> 3))
+        return MSD_ERR_INVALID_VALUE;
+    if (ranges_overlap(src, count * elt_bytes(dtype), dst, count * elt_bytes(dtype))) return MSD_ERR_INVALID_VALUE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == MSD_DTYPE_F32) return permute_021_dispatch<float>(src, dst, isize, jsize, ksize, s);
     return permute_021_dispatch<__half>(src, dst, isize, jsize, ksize, s);
@@ -423,7 +465,9 @@ int msd_linear_rows(const void *x, const void *weight, const float *bias, void *
         (act_out != MSD_ACT_NONE && act_out != MSD_ACT_SILU))
         return MSD_ERR_INVALID_VALUE;
     if (m > 8) return MSD_ERR_INVALID_VALUE;
-    if (m * n != 0 && (!y || (k != 0 && (!x || !weight)) || x == y)) return MSD_ERR_INVALID_VALUE;
+    if (m * n != 0 && (!y || (k != 0 && (!x || !weight)))) return MSD_ERR_INVALID_VALUE;
+    if (n > (SIZE_MAX >> 8) || k > (SIZE_MAX >> 8)) return MSD_ERR_INVALID_VALUE;
+    if (ranges_overlap(x, m * k * elt_bytes(dtype), y, m * n * elt_bytes(dtype))) return MSD_ERR_INVALID_VALUE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == MSD_DTYPE_F32)
         return linear_rows_dispatch<float>(x, weight, bias, y, m, n, k, act_in, act_out, s);
@@ -439,9 +483,12 @@ int msd_linear_rows_grouped(const void *x, const void *const *weights, const flo
         return MSD_ERR_INVALID_VALUE;
     if (m > 8) return MSD_ERR_INVALID_VALUE;
     if (count != 0 && (!weights || !ys || !ns)) return MSD_ERR_INVALID_VALUE;
+    if (k > (SIZE_MAX >> 8)) return MSD_ERR_INVALID_VALUE;
     for (size_t i = 0; i < count && m != 0; i++) {
         if (ns[i] == 0) continue;
-        if (!ys[i] || (k != 0 && (!x || !weights[i])) || x == ys[i]) return MSD_ERR_INVALID_VALUE;
+        if (!ys[i] || (k != 0 && (!x || !weights[i])) || ns[i] > (SIZE_MAX >> 8)) return MSD_ERR_INVALID_VALUE;
+        if (ranges_overlap(x, m * k * elt_bytes(dtype), ys[i], m * ns[i] * elt_bytes(dtype)))
+            return MSD_ERR_INVALID_VALUE;
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == MSD_DTYPE_F32)
@@ -453,6 +500,9 @@ int msd_softmax(const void *x, void *y, size_t rows, size_t cols, int stable, in
                 void *stream) {
     if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
     if (rows * cols != 0 && (!x || !y)) return MSD_ERR_INVALID_VALUE;
+    size_t count;
+    if (__builtin_mul_overflow(rows, cols, &count) || count > (SIZE_MAX >> 3)) return MSD_ERR_INVALID_VALUE;
+    if (shifted_overlap(x, y, count * elt_bytes(dtype))) return MSD_ERR_INVALID_VALUE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == MSD_DTYPE_F32) return softmax_dispatch<float>(x, y, rows, cols, stable != 0, s);
     return softmax_dispatch<__half>(x, y, rows, cols, stable != 0, s);
@@ -497,6 +547,9 @@ int msd_ddim_update(const void *x, const void *e_t, void *x_prev, size_t n, floa
     if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
     if (n != 0 && (!x || !e_t || !x_prev)) return MSD_ERR_INVALID_VALUE;
     if (!(a_t > 0.0f) || !(a_prev >= 0.0f) || !(a_prev <= 1.0f)) return MSD_ERR_INVALID_VALUE;  // sqrt / division
+    if (n > (SIZE_MAX >> 3) || shifted_overlap(x, x_prev, n * elt_bytes(dtype)) ||
+        shifted_overlap(e_t, x_prev, n * elt_bytes(dtype)))
+        return MSD_ERR_INVALID_VALUE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == MSD_DTYPE_F32)
         return ddim_update_dispatch<float>(x, e_t, x_prev, n, a_t, a_prev, sqrt_one_minus_at, s);

@@ -108,6 +108,54 @@ def test_argument_validation_needs_no_gpu(msd):
     assert lib.msd_ddim_schedule(501, None, None, None, None, 0) == -2
 
 
+def test_shifted_overlaps_are_refused_before_any_launch(msd):
+    """An output that may alias an input must be that input exactly or lie apart from it; an
+    output that must not overlap an input may not share a byte with it.  The addresses are
+    never dereferenced: every call below returns before anything is launched."""
+    lib = msd.load_library()
+    p = ctypes.c_void_p
+    base, w = 1 << 20, 1 << 24   # an activation range and a parameter range far away from it
+    f = ctypes.c_float
+    # [2, 64, 16] fp16 = 4096 bytes
+    gn = lambda x, y: lib.msd_groupnorm(p(x), p(y), p(w), p(w), 2, 64, 16, 32, f(1e-5), 1, 1, None)
+    assert gn(base, base + 2048) == 1 and gn(base + 4094, base) == 1
+    assert lib.msd_chunk_add_groupnorm(p(base), p(w), p(base + 64), p(w), p(w), 2, 64, 16, 32, f(1e-5), 1, 1, None) == 1
+    tok = lambda x, y: lib.msd_groupnorm_tokens(p(x), p(y), p(w), p(w), 2, 64, 16, 32, f(1e-6), 1, None)
+    assert tok(base, base) == 1 and tok(base, base + 4094) == 1 and tok(base + 2, base) == 1
+    # [8, 64] fp32 = 2048 bytes
+    ln = lambda x, y: lib.msd_layernorm(p(x), p(y), p(w), p(w), 8, 64, f(1e-5), 0, None)
+    assert ln(base, base + 4) == 1 and ln(base + 2044, base) == 1
+    addln = lambda a, b, s_, y: lib.msd_add_layernorm(p(a), p(b), p(s_), p(y), p(w), p(w), 8, 64, f(1e-5), 0, None)
+    far = base + (1 << 16)
+    assert addln(base, far, base + 8, far + 4096) == 1        # the sum shifted against a
+    assert addln(base, far, far + 8, far + 4096) == 1         # ... against b
+    assert addln(base, far, far + 4096, far + 4096) == 1      # the sum and the result in one place
+    assert addln(base, far, far + 4096, far + 4100) == 1
+    assert lib.msd_elemwise_add(p(base), p(far), p(base + 4), 512, 0, None) == 1
+    assert lib.msd_elemwise_add(p(base), p(far), p(far + 2044), 512, 0, None) == 1
+    assert lib.msd_chunkwise_add(p(base), p(w), p(base + 4), 512, 64, 0, None) == 1
+    assert lib.msd_chunkwise_add(p(base), p(base + 2048 + 16), p(base + 2048), 512, 64, 0, None) == 1  # chunk inside c
+    for act in (lib.msd_silu, lib.msd_gelu, lib.msd_quick_gelu):
+        assert act(p(base), p(base + 2), 512, 1, None) == 1
+    perm = lambda a, b: lib.msd_permute_0_2_1(p(a), p(b), 2, 16, 16, 1, None)   # 1024 bytes
+    assert perm(base, base) == 1 and perm(base, base + 1022) == 1 and perm(base + 512, base) == 1
+    # Linear: x [2, 8], y [2, 4] fp32
+    lin = lambda x, y: lib.msd_linear_rows(p(x), p(w), None, p(y), 2, 4, 8, 0, 0, 0, None)
+    assert lin(base, base) == 1 and lin(base, base + 60) == 1 and lin(base + 28, base) == 1
+    ys = (ctypes.c_void_p * 2)(far, base + 60)
+    ws = (ctypes.c_void_p * 2)(w, w)
+    ns = (ctypes.c_size_t * 2)(4, 4)
+    assert lib.msd_linear_rows_grouped(p(base), ws, None, ys, ns, 2, 2, 8, 0, 0, 0, None) == 1
+    assert lib.msd_softmax(p(base), p(base + 2), 4, 77, 0, 1, None) == 1
+    upd = lambda x, e, y: lib.msd_ddim_update(p(x), p(e), p(y), 64, f(0.5), f(0.6), f(0.7), 0, None)
+    assert upd(base, far, base + 4) == 1 and upd(base, far, far + 252) == 1
+    # sizes whose byte count does not fit are refused as well
+    huge = (1 << 62)
+    assert lib.msd_silu(p(base), p(far), huge, 0, None) == 1
+    assert lib.msd_permute_0_2_1(p(base), p(far), 1 << 31, 1 << 31, 8, 1, None) == 1
+    assert lib.msd_groupnorm(p(base), p(far), p(w), p(w), 1 << 40, 32, 1 << 30, 32, f(1e-5), 0, 0, None) == 1
+
+
 def test_missing_library_fails_loudly(msd):
     with pytest.raises(msd.MsdError):
         msd.load_library(os.path.join(REPO, "does_not_exist.so"))
