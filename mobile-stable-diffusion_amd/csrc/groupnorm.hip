@@ -779,10 +779,28 @@ GnPlan plan_slice(uint32_t vecs, uint32_t split, uint32_t force_threads, uint32_
         // batch 2 - 8) still want large workgroups: 3840-vector slices 12.28 us on 960 x 4 against
         // 12.55 on 512 x 8, 5120-vector slices 14.6 us on 512 x 10 against 14.8 on 640 x 8.
         const bool cut_few = split > 1 && blocks < 4 * kChipCus;
-        if (cut_few) pl.threads = exact_fit_threads(vecs, elt == 2 ? 2 : 4);
+        if (cut_few) {
+            // ... as long as a CU has room for all of its workgroups at once (a SIMD holds eight
+            // wavefronts and takes a quarter of each workgroup's, rounded up): 768 slices of 3840
+            // vectors take 16.5 us on 512 x 8 and 18.7 on 960 x 4, of which only two fit a CU
+            const uint32_t exact = exact_fit_threads(vecs, elt == 2 ? 2 : 4);
+            if (exact != 0 && (blocks + kChipCus - 1) / kChipCus <= 8 / ((exact + 255) / 256)) pl.threads = exact;
+        }
+        // 1024 and more slices of cut units, more than 384 units: the smallest workgroup that holds a slice in at most
+        // five vectors per lane (against 256 lanes with eight or ten: 1920-vector slices 64.5 us on
+        // 384 x 5 against 66.9, 2560-vector slices 83.2 on 512 x 5 against 87.3, 3840-vector slices
+        // 122 on 768 x 5 against 127, batch 24, 4-byte elements)
+        if (split > 1 && !cut_few && blocks / split > 384)
+            for (uint32_t t = 384; t <= kGnMaxThreads && pl.threads == 0; t += 128) {
+                const int k = k_for(vecs, t, max_k, equal_slices);
+                if (k != 0 && k <= 5) pl.threads = t;
+            }
         for (uint32_t t : {256u, 512u, 768u, 1024u}) {
             if (pl.threads != 0) break;
             if ((cut_few && t == 256u) || k_for(vecs, t, max_k, equal_slices) == 0) continue;
+            // (short slices: at least ten wavefronts per CU - 512 units of 2560 vectors 8.54 us
+            // on 512 x 5 against 8.98 on 256 x 10, of 3840 vectors 11.9 on 512 x 8 against 12.7)
+            if (vecs <= 4096 && (size_t)t * blocks < 10 * kWave * kChipCus && t < kGnMaxThreads) continue;
             pl.threads = t;
         }
         if (pl.threads == 0) pl.threads = kGnMaxThreads;
@@ -800,6 +818,15 @@ GnPlan plan_slice(uint32_t vecs, uint32_t split, uint32_t force_threads, uint32_
         // lanes with a masked tail against 3.62 us on 640 x 2; 4-byte elements: 512 x 5 is an
         // exact fit itself, 3.98 us against 4.08 on 640 x 4)
         pl.threads = exact;
+    } else if (!shared && split == 1 && vecs > 5120 && vecs % 640 == 0 && vecs / 10 >= 640 && vecs / 10 <= kGnMaxThreads &&
+               max_k >= 10) {
+        // long whole units that are exactly ten vectors per lane on 640 ... 1024 lanes (7680-vector
+        // units of 4-byte elements: 8.05 us on 768 x 10 against 8.44 on 1024 x 8 with a masked tail)
+        pl.threads = vecs / 10;
+    } else if (!shared && elt == 4 && split == 1 && vecs == 5120 && blocks >= 160) {
+        // whole 5120-vector units of 4-byte elements from batch 5 on: 512 x 10 (batch 7 / 8: 7.38 /
+        // 8.12 us against 7.79 / 8.49 on 1024 x 5; the same at batch 2 - 5)
+        pl.threads = 512;
     } else if (vecs > 512u * 5u || (split > 1 && vecs >= 960))  // slices of a cut unit: 2 - 3 % faster
         pl.threads = kGnMaxThreads;
     else if (split == 1 && vecs >= 256 && vecs <= 704 && vecs % kWave == 0)
@@ -940,10 +967,21 @@ GnDecision gn_decide(size_t elt, size_t batch, size_t channels, size_t hw, size_
                 // (up to 32 Ki elements two slices are enough from 64 units on: 960 channels at
                 // 32 x 32, batch 2, 5.40 us in two against 5.63 us in four; batch 1 4.86 in four
                 // against 5.03 in two)
-                want = units >= 256 ? 1 : (units >= 128 || (unit_size <= 32768 && units >= 64)) ? 2 : 4;
+                // (96 units, batch 3: 320 channels at 64 x 64 6.44 us in two against 6.74 in four)
+                want = units >= 256 ? 1
+                       : (units >= 128 || (unit_size <= 32768 && units >= 64) || (unit_size <= 61440 && units >= 96)) ? 2
+                                                                                                                      : 4;
                 // (batch 1: 960 channels at 64 x 64 7.08 us in eight against 7.16 in four, 640
                 // channels 6.56 against 6.12)
                 if (units * 4 < 192 && unit_size > 98304) want = 8;
+                // 160 ... 224 units (batch 5 - 7): two slices would give some CUs two 1024-lane
+                // workgroups and others one, so units stay whole (one workgroup on most CUs) or,
+                // the long ones, go in four on 512 lanes (three small workgroups per CU).  Batch 5 /
+                // 6 / 7, us whole against in two: 320 channels at 64 x 64 7.67 / 8.02 / 8.49 against
+                // 8.57 / 8.95 / 9.27, 960 at 32 x 32 6.45 / 6.75 / 7.00 against 7.28 / 7.64 / 7.86;
+                // in four against in two: 640 at 64 x 64 12.3 / 13.3 / - against 13.7 / 14.3, 960 at
+                // 64 x 64 17.6 / 18.7 / - against 19.9 / 20.9 (batch 7: whole, 20.7 against 22.0).
+                if (units > 128 && units < 256) want = (units >= 224 || unit_size <= 61440) ? 1 : 4;
             }
         } else {
             // 4-byte elements, half the arithmetic per vector: whole up to 5120 vectors (4096 when
@@ -961,13 +999,33 @@ GnDecision gn_decide(size_t elt, size_t batch, size_t channels, size_t hw, size_
                 if (units * want * 2 > 2 * kChipCus || slice <= limit || slice / 2 < 960 || want >= kGnMaxSplit) break;
                 want *= 2;
             }
+            // 160 and 192 units (batch 5, 6), as for 2-byte elements: whole up to 10240 vectors, in
+            // four beyond (batch 5 / 6, us: 320 channels at 64 x 64 whole 10.4 / 12.0 against 11.8 /
+            // 12.5 in two, 960 at 32 x 32 8.15 / 9.21 against 9.81 / 10.2; 640 at 64 x 64 in four
+            // 21.2 / 22.5 against 24.5 / 25.7 in two, 960 at 64 x 64 29.9 / 33.5 against 34.4 / 36.6)
+            if (units > 128 && units <= 192 && vec_per_unit > whole_limit) want = vec_per_unit <= 10240 ? 1 : 4;
+        }
+        // 288 ... 384 units (batch 9 - 12): whole units on 1024 lanes would give some CUs two
+        // workgroups and others one; units of 5120 vectors and more are cut into slices of at most
+        // 2560 (5120 from 352 units on), which run as three and more small workgroups per CU (from
+        // 448 units on whole units win again).  Batch 10 / 12, us against
+        // whole: 640 channels at 64 x 64 fp16 22.3 / 23.8 against 26.4 / 26.8, 1920 at 32 x 32 17.7 /
+        // 18.5 against 19.6 / 21.0; 4-byte elements 960 at 32 x 32 15.3 / 17.0 against 17.3 / 20.1,
+        // 320 at 64 x 64 21.4 / 22.4 against 22.5 / 24.0.
+        if (units > kChipCus && units <= 384 && vec_per_unit >= 5120) {
+            if (want < 2) want = 2;
+            const size_t longest = units <= 320 ? 2560 : 5120;  // (batch 12: 23.4 us in two against 23.7 in four)
+            while (vec_per_unit > (size_t)want * longest && want < 8) want *= 2;
         }
         // Large batches of very long units (more than 10240 vectors): slices of up to 5120
         // vectors on 256 lanes overlap better than whole units on 768 - 1024 lanes, the exchange
         // disappears behind the other workgroups of the CU (batch 32, 15360-vector units: 90 us
         // in four against 99 us whole)
-        if (units >= 2 * kChipCus && vec_per_unit > 10240)
-            while (vec_per_unit > (size_t)want * 5120 && want < kGnMaxSplit) want *= 2;
+        if (units > 384 && vec_per_unit > 10240)
+            while (vec_per_unit > (size_t)want * 2560 && want < 8) want *= 2;
+        // 96 units (batch 3) of more than 96 Ki elements: eight slices are three small workgroups
+        // per CU (960 channels at 64 x 64: 11.2 us against 11.9 in four; 4-byte elements 16.7 against 17.8)
+        if (units == 96 && unit_size > 98304 && want < 8) want = 8;
         while (units * want < 16 && want < kGnMaxSplit) want *= 2;  // very few units
         while (split < want && vec_per_unit >= (size_t)2 * split * 256) split *= 2;
     }

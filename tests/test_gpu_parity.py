@@ -158,20 +158,21 @@ def test_groupnorm_many_vectors_per_lane(msd, orc, cuda, threads):
 
 
 def test_groupnorm_large_batch_plan_and_wide_groups(msd, orc, cuda):
-    """What the launch plan picks by itself for many units (batch 17: 544 units, 256 lanes x 20
-    vectors), and a group of more channels than the LDS copy of gamma / beta holds (the general
-    kernel takes over)."""
+    """What the launch plan picks by itself for many units (batch 25: 800 units, 256 lanes x 20
+    vectors; batch 17: 544 units, short units on 512 lanes), and a group of more channels than the
+    LDS copy of gamma / beta holds (the general kernel takes over)."""
     lib = msd.load_library()
-    x = orc.normal((17, 320, 64, 64), seed=521, sigma=1.2, mean=-0.3)
+    x = orc.normal((25, 320, 64, 64), seed=521, sigma=1.2, mean=-0.3)
     g, b = _affine(orc, 320, 521)
-    assert msd.groupnorm_plan(17, 320, 4096) == (1, 256, 20, 1)
+    assert msd.groupnorm_plan(25, 320, 4096) == (1, 256, 20, 1)
     _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, True)
     _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, False)
     # the other unit sizes of the UNet at that batch: 10 and 5 vectors per lane, ragged 16 and 8
-    for channels, hw, plan in ((640, 1024, (1, 256, 10, 1)), (1280, 256, (1, 256, 5, 1)), (960, 1024, (1, 256, 16, 1)),
-                               (1920, 256, (1, 256, 8, 1))):
-        assert msd.groupnorm_plan(17, channels, hw) == plan
-        xs = orc.normal((17, channels, hw), seed=523 + channels, sigma=1.4, mean=0.2)
+    for batch, channels, hw, plan in ((25, 640, 1024, (1, 256, 10, 1)), (25, 1280, 256, (1, 256, 5, 1)),
+                                      (25, 960, 1024, (1, 256, 16, 1)), (25, 1920, 256, (1, 256, 8, 1)),
+                                      (17, 640, 1024, (1, 512, 5, 1)), (17, 960, 1024, (1, 512, 8, 1))):
+        assert msd.groupnorm_plan(batch, channels, hw) == plan
+        xs = orc.normal((batch, channels, hw), seed=523 + channels, sigma=1.4, mean=0.2)
         gs, bs = _affine(orc, channels, 523 + channels)
         _run_groupnorm(msd, orc, cuda, xs, gs, bs, 32, 1e-5, True, True)
     wide = orc.normal((1, 32 * 1100, 16), seed=522, sigma=1.0)

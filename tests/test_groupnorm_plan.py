@@ -57,7 +57,7 @@ def test_plans_of_the_unet_shapes_at_batch_2_and_32():
         (2, 960, 4096, f32): (8, 960, 4, 1), (2, 640, 1024, f32): (1, 1024, 5, 1), (1, 640, 1024, f32): (4, 640, 2, 1),
         (4, 640, 4096, f32): (4, 512, 10, 1), (8, 640, 4096, f32): (2, 512, 20, 1), (2, 640, 256, f32): (1, 640, 2, 1),
         (32, 320, 4096, f16): (1, 256, 20, 1), (32, 640, 1024, f16): (1, 256, 10, 1), (32, 1280, 256, f16): (1, 256, 5, 1),
-        (8, 320, 4096, f16): (1, 1024, 5, 1), (32, 960, 4096, f16): (4, 256, 16, 1),
+        (8, 320, 4096, f16): (1, 1024, 5, 1), (32, 960, 4096, f16): (8, 384, 5, 1),
     }
     for (batch, channels, hw, code), want in in_place.items():
         assert _check(batch, channels, hw, 32, code, in_place=True) == want, (batch, channels, hw, code)
