@@ -51,7 +51,7 @@ def rnd_hw():
 
 def gn_case():
     groups = int(rng.choice([1, 2, 4, 8, 32])); cpg = int(rng.integers(1, 13)); C = groups * cpg
-    batch = int(rng.choice([1, 2, 3, 4, 8, 12, 17, 40])); hw = rnd_hw(); half = bool(rng.integers(0, 2)); silu = bool(rng.integers(0, 2))
+    batch = int(rng.choice([1, 2, 3, 4, 5, 6, 8, 10, 12, 17, 40])); hw = rnd_hw(); half = bool(rng.integers(0, 2)); silu = bool(rng.integers(0, 2))
     if batch * C * hw > 6e6: hw = max(1, int(6e6 // (batch * C)))
     # now and then a forced launch plan (workgroup size, slices per unit); refused values are ignored
     lib = msd.load_library()
