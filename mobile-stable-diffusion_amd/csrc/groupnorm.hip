@@ -1168,8 +1168,16 @@ int gn_tokens_dispatch(const void *xv, void *yv, const float *gamma, const float
     // share an XCD, which is worth more than the exchange costs from 16 Ki elements on)
     uint32_t want = 1;
     if (unit_size > 16384) {
-        want = units >= 256 ? 1 : units >= 128 ? 2 : 4;
-        if (units * 4 < 192 && unit_size >= 65536) want = 8;
+        // (more than 128 units: two slices would put two large workgroups on some CUs and one on
+        // others - 640 channels at 32 x 32, batch 5 / 6 / 7: 8.80 / 9.15 / 9.80 us whole against
+        // 9.56 / 10.2 / 10.6 in two)
+        want = units > 128 ? 1 : units >= 128 ? 2 : 4;
+        // (batch 1, 320 channels at 64 x 64: 6.59 us in eight against 7.16 in four, 4-byte elements
+        // 7.45 against 8.45)
+        if (units * 4 < 192 && unit_size >= 32768) want = 8;
+        // (288 and 320 units of 32 Ki elements and more: batch 10, 320 channels at 64 x 64 25.2 us
+        // in four against 29.4 whole; from 384 units on whole units win)
+        if (units > 256 && units <= 320 && unit_size >= 32768) want = 4;
     }
     const int tune_split = g_tuning.gn_split.load(std::memory_order_relaxed);
     const int tune_spin = g_tuning.gn_spin_limit.load(std::memory_order_relaxed);
