@@ -47,6 +47,22 @@ def _check(batch, channels, hw, groups, code, noalloc=False, in_place=False):
     return split, threads, k, writers
 
 
+def test_plans_at_the_batches_in_between():
+    """Between one and two workgroups per CU the plan keeps units whole or cuts them into many small
+    slices, never into one to two 1024-lane workgroups per CU (the measured rules of gn_decide)."""
+    f16, f32 = msd.DTYPE_F16, msd.DTYPE_F32
+    in_place = {
+        (3, 320, 4096, f16): (2, 1024, 3, 1), (3, 960, 4096, f16): (8, 512, 4, 1),
+        (5, 320, 4096, f16): (1, 1024, 5, 1), (6, 640, 4096, f16): (4, 512, 5, 1), (7, 960, 4096, f16): (1, 1024, 16, 1),
+        (5, 960, 1024, f32): (1, 768, 10, 1), (6, 1920, 1024, f32): (4, 512, 8, 1), (7, 640, 1024, f32): (1, 512, 10, 1),
+        (10, 640, 4096, f16): (4, 256, 10, 1), (12, 640, 4096, f16): (2, 512, 10, 1), (10, 320, 4096, f32): (4, 256, 10, 1),
+        (14, 320, 4096, f16): (1, 1024, 5, 1), (16, 640, 1024, f16): (1, 512, 5, 1), (24, 640, 4096, f32): (8, 512, 5, 1),
+        (24, 640, 1024, f16): (1, 256, 10, 1),
+    }
+    for (batch, channels, hw, code), want in in_place.items():
+        assert _check(batch, channels, hw, 32, code, in_place=True) == want, (batch, channels, hw, code)
+
+
 def test_plans_of_the_unet_shapes_at_batch_2_and_32():
     f16, f32 = msd.DTYPE_F16, msd.DTYPE_F32
     # a call in place (the reference's out-norms): one workgroup per unit or slices with an exchange
