@@ -157,6 +157,23 @@ def test_groupnorm_many_vectors_per_lane(msd, orc, cuda, threads):
     assert msd.status() == 0
 
 
+@pytest.mark.parametrize("batch,channels,hw,half,plan", [
+    (3, 320, 4096, True, (2, 1024, 3, 1)), (3, 960, 4096, True, (8, 512, 4, 1)), (5, 320, 4096, True, (1, 1024, 5, 1)),
+    (6, 640, 4096, True, (4, 512, 5, 1)), (5, 960, 1024, False, (1, 768, 10, 1)), (6, 1920, 1024, False, (4, 512, 8, 1)),
+    (7, 640, 1024, False, (1, 512, 10, 1)), (10, 640, 4096, True, (4, 256, 10, 1)), (12, 640, 4096, True, (2, 512, 10, 1)),
+    (10, 320, 4096, False, (4, 256, 10, 1)), (16, 640, 1024, True, (1, 512, 5, 1))])
+def test_groupnorm_plans_at_the_batches_in_between(msd, orc, cuda, batch, channels, hw, half, plan):
+    """The launches the plan makes between one and two workgroups per CU (whole units or many
+    small slices), in place as the reference's out-norms run and out of place."""
+    code = msd.DTYPE_F16 if half else msd.DTYPE_F32
+    assert msd.groupnorm_plan(batch, channels, hw, 32, code, False, True) == plan
+    x = orc.normal((batch, channels, hw), seed=batch * 1000 + channels, sigma=1.3, mean=0.4)
+    g, b = _affine(orc, channels, batch + channels)
+    _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half, inplace=True)
+    _run_groupnorm(msd, orc, cuda, x, g, b, 32, 1e-5, True, half)
+    assert msd.status() == 0
+
+
 def test_groupnorm_large_batch_plan_and_wide_groups(msd, orc, cuda):
     """What the launch plan picks by itself for many units (batch 25: 800 units, 256 lanes x 20
     vectors; batch 17: 544 units, short units on 512 lanes), and a group of more channels than the
