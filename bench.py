@@ -7,8 +7,10 @@ the timestep embedding, 23 SiLU(emb), 45 GroupNorm(32)+SiLU (in- and out-norm of
 each layer on its own HBM-resident buffers, launched back to back on one stream.
 `value` = algorithmic bytes of one step / time per step.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode graph|eager]
-                    [--no-cpu] [--no-shapes] [--tables shapes,fusions,neighbours,large_batch,gn_split]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode graph|eager] [--no-cpu] [--no-shapes]
+                    [--tables shapes,gn_split,fusions,neighbours,large_batch,gn_plan_sweep]
+    python bench.py --sweep-summary OUT.json[,...]               (no GPU: markdown of gn_plan_sweep rows)
+    python bench.py --trace-summary TRACE.csv --bench-json OUT   (no GPU: shapes rows next to a kernel trace)
 
 Prints ONE JSON line (see the keys below).  The CPU oracle is used only for the
 `cpu_baseline` leg.
@@ -266,20 +268,74 @@ def _rotating_launch_us(torch, msd, stream, launch, xs, ys, warm=20, budget=2000
         return event_time_ms(torch, replay, reps) * 1e3 / (reps * copies)
 
 
-def _gn_plan_text(msd, batch, channels, hw, elt):
+_HIP_RUNTIME = None
+
+
+def hip_runtime():
+    """ctypes handle of the HIP runtime this process already uses (the copy torch loaded, found
+    in /proc/self/maps so that no second runtime is mapped), with hipMemcpyDtoDAsync declared."""
+    global _HIP_RUNTIME
+    if _HIP_RUNTIME is None:
+        import ctypes
+        path = None
+        with open("/proc/self/maps") as f:
+            for line in f:
+                name = line.split()[-1]
+                if "/libamdhip64.so" in name:
+                    path = name
+                    break
+        if path is None:
+            raise RuntimeError("the HIP runtime is not mapped into this process")
+        rt = ctypes.CDLL(path)
+        rt.hipMemcpyDtoDAsync.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        rt.hipMemcpyDtoDAsync.restype = ctypes.c_int
+        _HIP_RUNTIME = rt
+    return _HIP_RUNTIME
+
+
+class TraceMarkers:
+    """Numbers the timed measurements of a table so that a kernel trace of the same run can be cut
+    into them: before measurement i one tiny launch of a kernel no table uses (quick_GELU on fp16)
+    with i + 1 workgroups goes onto the stream; `labels[i]` says what was measured after it."""
+
+    def __init__(self, torch, msd, dev):
+        import ctypes
+        self.labels = []
+        self._lib = msd.load_library()
+        self._code = msd.DTYPE_F16
+        self._vp = ctypes.c_void_p
+        self._torch = torch
+        self._buf = torch.zeros(512 * 256 * 8, device=dev, dtype=torch.float16)  # room for 512 markers
+
+    def mark(self, label):
+        i = len(self.labels)
+        n = (i + 1) * 256 * 8  # i + 1 workgroups of 256 lanes, one 16-byte vector per lane
+        if n > self._buf.numel():
+            raise RuntimeError("too many trace markers")
+        p = self._vp(self._buf.data_ptr())
+        sp = self._vp(self._torch.cuda.current_stream().cuda_stream)
+        assert self._lib.msd_quick_gelu(p, p, n, self._code, sp) == 0
+        self._torch.cuda.synchronize()
+        self.labels.append(label)
+
+
+def _gn_plan_text(msd, batch, channels, hw, elt, in_place=False):
     """'slices per unit x lanes x vectors per lane' of the GroupNorm launch for this shape (output
-    apart from the input, as the tables run it), ', w writers' when w workgroups share each whole
-    unit and store a w-th of it each."""
+    apart from the input unless in_place), ', w writers' when w workgroups share each whole unit
+    and store a w-th of it each."""
     split, threads, k, writers = msd.groupnorm_plan(batch, channels, hw, 32,
-                                                    msd.DTYPE_F16 if elt == 2 else msd.DTYPE_F32)
+                                                    msd.DTYPE_F16 if elt == 2 else msd.DTYPE_F32,
+                                                    in_place=in_place)
     if split == 0:
         return "general kernel"
     text = "%d x %d lanes x %d vectors" % (split, threads, k)
     return text + (", %d writers" % writers if writers > 1 else "")
 
 
-def _kernel_case(torch, msd, dev, kind, p, dt, batch):
-    """Buffers, launch closure and byte counts for one row of the per-kernel tables."""
+def _kernel_case(torch, msd, dev, kind, p, dt, batch, sigma=1.0):
+    """Buffers, launch closures and byte counts for one row of the per-kernel tables; inputs are
+    N(0, sigma).  `launch(x, y, stream)` writes y apart from x; GroupNorm is also timed with
+    y == x (launch(x, x, stream)), the form of the reference's out-norms (M/nn/ResBlock.cpp:222)."""
     import ctypes
     vp = ctypes.c_void_p
     lib = msd.load_library()
@@ -297,7 +353,7 @@ def _kernel_case(torch, msd, dev, kind, p, dt, batch):
         n_in = n_out = p["n"]
         nbytes = 2 * n_in * elt
     copies = max(4, min(256, int(640e6 // max(nbytes, 1)) + 1))
-    xs = [torch.randn(n_in, device=dev, dtype=torch.float32).to(dt) for _ in range(copies)]
+    xs = [(torch.randn(n_in, device=dev, dtype=torch.float32) * sigma).to(dt) for _ in range(copies)]
     ys = [torch.empty(n_out, device=dev, dtype=dt) for _ in range(copies)]
     cdim = p.get("c", p.get("dim", 1))
     ga = torch.ones(cdim, device=dev)
@@ -325,42 +381,87 @@ def _kernel_case(torch, msd, dev, kind, p, dt, batch):
             "bytes": nbytes, "copy_same_bytes": True, "elt": elt}
 
 
-def shape_table(torch, msd, dev, stream):
-    """Per-kernel µs / GB/s / % of HBM peak at the shapes of BASELINE configs 1 - 4, each launch
-    on its own buffers (rotating over > 600 MB so nothing is cache-resident), graph-replayed,
-    next to a plain copy of the same bytes.  Config 2 / 3 at batch 2 in fp16 (GroupNorm also
-    fp32); config 1 (one fp32 tensor) and config 4 (text-encoder shapes, fp32) are a few hundred
-    KB to 10 MB per launch and are bound by the launch floor, not by bandwidth."""
+def shape_cases(torch):
+    """(config, kernel, shape, dtype, batch, sigma of the N(0, sigma) input) of the per-kernel
+    table: the shapes of BASELINE configs 1 - 4 (config 2 draws x from N(0, 2))."""
     f16, f32 = torch.float16, torch.float32
-    cases = [("cfg1", "groupnorm_silu", {"c": 320, "hw": 4096}, f32, 1)]
+    cases = [("cfg1", "groupnorm_silu", {"c": 320, "hw": 4096}, f32, 1, 1.0)]
     for c, side in [(320, 64), (640, 32), (1280, 16), (1280, 8), (960, 32), (1920, 16)]:
-        cases.append(("cfg2", "groupnorm_silu", {"c": c, "hw": side * side}, f16, BATCH))
-        cases.append(("cfg2", "groupnorm_silu", {"c": c, "hw": side * side}, f32, BATCH))
+        cases.append(("cfg2", "groupnorm_silu", {"c": c, "hw": side * side}, f16, BATCH, 2.0))
+        cases.append(("cfg2", "groupnorm_silu", {"c": c, "hw": side * side}, f32, BATCH, 2.0))
     for r, d in [(8192, 320), (2048, 640), (512, 1280)]:
-        cases.append(("cfg3", "layernorm", {"rows": r, "dim": d}, f16, BATCH))
+        cases.append(("cfg3", "layernorm", {"rows": r, "dim": d}, f16, BATCH, 1.0))
     for r, i in [(8192, 1280), (2048, 2560), (512, 5120)]:
-        cases.append(("cfg3", "geglu", {"rows": r, "inner": i}, f16, BATCH))
-    cases.append(("cfg4", "layernorm", {"rows": 77, "dim": 768}, f32, 1))
-    cases.append(("cfg4", "layernorm", {"rows": 154, "dim": 768}, f32, 2))
-    cases.append(("cfg4", "quick_gelu", {"n": 2 * 77 * 3072}, f32, 2))
+        cases.append(("cfg3", "geglu", {"rows": r, "inner": i}, f16, BATCH, 1.0))
+    cases.append(("cfg4", "layernorm", {"rows": 77, "dim": 768}, f32, 1, 1.0))
+    cases.append(("cfg4", "layernorm", {"rows": 154, "dim": 768}, f32, 2, 1.0))
+    cases.append(("cfg4", "quick_gelu", {"n": 2 * 77 * 3072}, f32, 2, 1.0))
+    return cases
+
+
+def shape_table(torch, msd, dev, stream, floor_us, markers=None):
+    """Per-kernel µs / GB/s / % of HBM peak at the shapes of BASELINE configs 1 - 4, each launch
+    on its own buffers (rotating over > 600 MB so nothing is cache-resident), graph-replayed.
+    Config 2 / 3 at batch 2 in fp16 (GroupNorm also fp32); config 1 (one fp32 tensor) and config 4
+    (text-encoder shapes, fp32) are a few hundred KB to 10 MB per launch and are bound by the
+    launch floor, not by bandwidth.
+
+    Three yardsticks stand beside every row: `copy_us`, this library's plain 16-byte copy kernel
+    over the same bytes; `memcpy_us`, the HIP runtime's own device-to-device copy of the same
+    bytes (hipMemcpyDtoDAsync, captured as memcpy nodes and replayed like everything else);
+    `floor_model_us` = the launch floor of a graph node + bytes / 8 TB/s.  GroupNorm rows carry
+    `us` / `plan` for an output apart from the input and `us_in_place` / `plan_in_place` for
+    y == x (the reference's out-norms, M/nn/ResBlock.cpp:222, where no two workgroups may share a
+    unit).  `frac_hbm_peak*` = bytes / time / 8 TB/s."""
+    import ctypes
+    vp = ctypes.c_void_p
+    rt = hip_runtime()
     rows = []
-    for cfg, kind, p, dt, batch in cases:
-        case = _kernel_case(torch, msd, dev, kind, p, dt, batch)
-        us = _rotating_launch_us(torch, msd, stream, case["launch"], case["xs"], case["ys"])
-        gbs = case["bytes"] / us / 1e3
+
+    def mark(row, what):
+        if markers is not None:
+            markers.mark({"row": len(rows), "what": what, "kernel": row["kernel"], "shape": row["shape"],
+                          "dtype": row["dtype"], "bytes": row["bytes"]})
+
+    for cfg, kind, p, dt, batch, sigma in shape_cases(torch):
+        case = _kernel_case(torch, msd, dev, kind, p, dt, batch, sigma)
+        nbytes = case["bytes"]
         row = {"config": cfg, "kernel": kind, "shape": dict(p, batch=batch), "dtype": "f16" if case["elt"] == 2 else "f32",
-               "bytes": case["bytes"], "us": round(us, 3), "GBps": round(gbs, 1),
-               "pct_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 1)}
-        if case["copy_same_bytes"]:  # one copy launch moves exactly the kernel's bytes
-            cus = _rotating_launch_us(torch, msd, stream, case["copy_launch"], case["xs"], case["ys"])
-            row["copy_us"] = round(cus, 3)
-            row["pct_of_copy_rate"] = round(100.0 * cus / us, 1)
-        if cfg in ("cfg1", "cfg4"):
-            row["note"] = "launch-bound: %.2f us at 8 TB/s" % (case["bytes"] / HBM_PEAK_GBS / 1e3)
+               "bytes": nbytes}
+        mark(row, "us")
+        us = _rotating_launch_us(torch, msd, stream, case["launch"], case["xs"], case["ys"])
+        gbs = nbytes / us / 1e3
+        row.update({"us": round(us, 3), "GBps": round(gbs, 1), "pct_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 1),
+                    "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)})
         if kind == "groupnorm_silu":
             row["plan"] = _gn_plan_text(msd, batch, p["c"], p["hw"], case["elt"])
+            mark(row, "us_in_place")
+            ius = _rotating_launch_us(torch, msd, stream, lambda x, y, sp: case["launch"](x, x, sp), case["xs"],
+                                      case["ys"])
+            row["us_in_place"] = round(ius, 3)
+            row["frac_hbm_peak_in_place"] = round(nbytes / ius / 1e3 / HBM_PEAK_GBS, 4)
+            row["plan_in_place"] = _gn_plan_text(msd, batch, p["c"], p["hw"], case["elt"], in_place=True)
+        mark(row, "copy_us")
+        cus = _rotating_launch_us(torch, msd, stream, case["copy_launch"], case["xs"], case["ys"])
+        row["copy_us"] = round(cus, 3)
+        row["pct_of_copy_rate"] = round(100.0 * cus / us, 1)
+        copy_dst = case["keep"][2]
+
+        def memcpy_launch(x, y, sp):  # the runtime's own copy of the same bytes (half read, half written)
+            dst = copy_dst.get(x.data_ptr(), y)
+            return rt.hipMemcpyDtoDAsync(vp(dst.data_ptr()), vp(x.data_ptr()), nbytes // 2, sp)
+        mark(row, "memcpy_us")
+        mus = _rotating_launch_us(torch, msd, stream, memcpy_launch, case["xs"], case["ys"])
+        row["memcpy_us"] = round(mus, 3)
+        row["pct_of_memcpy_rate"] = round(100.0 * mus / us, 1)
+        row["floor_model_us"] = round(floor_us + nbytes / HBM_PEAK_GBS / 1e3, 3)
+        if "us_in_place" in row:
+            row["pct_of_copy_rate_in_place"] = round(100.0 * cus / row["us_in_place"], 1)
+            row["pct_of_memcpy_rate_in_place"] = round(100.0 * mus / row["us_in_place"], 1)
+        if cfg in ("cfg1", "cfg4"):
+            row["note"] = "launch-bound: %.2f us at 8 TB/s" % (nbytes / HBM_PEAK_GBS / 1e3)
         rows.append(row)
-        del case
+        del case, copy_dst
         torch.cuda.empty_cache()
     return rows
 
@@ -396,7 +497,7 @@ def gn_split_table(torch, msd, dev, stream):
     rows = []
     for c, side in [(320, 64), (640, 32), (1280, 16), (1280, 8), (960, 32), (1920, 16)]:
         for dt in (torch.float16, torch.float32):
-            case = _kernel_case(torch, msd, dev, "groupnorm_silu", {"c": c, "hw": side * side}, dt, BATCH)
+            case = _kernel_case(torch, msd, dev, "groupnorm_silu", {"c": c, "hw": side * side}, dt, BATCH, 2.0)
             times = {}
             try:
                 assert lib.msd_set_tuning(msd.TUNE_GN_WRITERS, 0) == 0
@@ -422,6 +523,183 @@ def gn_split_table(torch, msd, dev, stream):
             del case
             torch.cuda.empty_cache()
     return rows
+
+
+def unet_gn_shapes():
+    """The distinct (channels, side) of the GroupNorms of one UNet step (in- and out-norms of the 22
+    ResBlocks; the final norm repeats one of them): 14 shapes."""
+    seen = []
+    for cin, cout, side in RESBLOCKS:
+        for c in (cin, cout):
+            if (c, side) not in seen:
+                seen.append((c, side))
+    return sorted(seen, key=lambda cs: (cs[0] * cs[1] * cs[1], cs[0]))
+
+
+SWEEP_THREADS = (256, 384, 512, 640, 768, 960, 1024)
+
+
+def gn_plan_sweep(torch, msd, dev, stream, batches, progress=None):
+    """GroupNorm+SiLU at the 14 GroupNorm shapes of the UNet x {fp16, fp32} x `batches` x {in place,
+    output apart}: the automatic launch plan timed against every plan the knobs can force
+    (1 / 2 / 4 / 8 slices per unit x 256 ... 1024 lanes, and for an output apart from the input also
+    2 / 4 / 8 writers per whole unit x the same workgroup sizes).  A forced setting counts only if
+    msd_groupnorm_plan confirms that the launch follows it; identical plans are timed once.  The
+    automatic plan and the fastest forced one are then timed twice more, alternating, and
+    `auto_vs_best` is the ratio of the medians: above 1.03 the planner picked a slow variant."""
+    lib = msd.load_library()
+    knobs = (msd.TUNE_GN_SPLIT, msd.TUNE_GN_THREADS, msd.TUNE_GN_WRITERS)
+
+    def set_knobs(split, threads, writers):
+        for knob, value in zip(knobs, (split, threads, writers)):
+            assert lib.msd_set_tuning(knob, value) == 0
+
+    def text(plan):
+        return "%dx%dx%d" % plan[:3] + (" w%d" % plan[3] if plan[3] > 1 else "")
+
+    rows = []
+    for batch in batches:
+        for c, side in unet_gn_shapes():
+            hw = side * side
+            for dt, code, elt in ((torch.float16, msd.DTYPE_F16, 2), (torch.float32, msd.DTYPE_F32, 4)):
+                case = _kernel_case(torch, msd, dev, "groupnorm_silu", {"c": c, "hw": hw}, dt, batch, 2.0)
+                budget = int(min(3000, max(300, 20000.0 / max(3.0, case["bytes"] / 4e6))))
+                for in_place in (True, False):
+                    launch = (lambda x, y, sp: case["launch"](x, x, sp)) if in_place else case["launch"]
+
+                    def timed():
+                        return _rotating_launch_us(torch, msd, stream, launch, case["xs"], case["ys"], budget=budget)
+                    try:
+                        set_knobs(0, 0, 0)
+                        auto_plan = msd.groupnorm_plan(batch, c, hw, 32, code, in_place=in_place)
+                        times = {auto_plan: timed()}
+                        for writers in ((1,) if in_place else (1, 2, 4, 8)):
+                            for split in ((1, 2, 4, 8) if writers == 1 else (1,)):
+                                for threads in SWEEP_THREADS:
+                                    set_knobs(split, threads, writers)
+                                    plan = msd.groupnorm_plan(batch, c, hw, 32, code, in_place=in_place)
+                                    if plan in times or plan[0] != split or plan[1] != threads or plan[3] != writers:
+                                        continue
+                                    times[plan] = timed()
+                        best_plan = min((pl for pl in times if pl != auto_plan), key=lambda pl: times[pl],
+                                        default=auto_plan)
+                        auto_runs, best_runs = [times[auto_plan]], [times[best_plan]]
+                        if best_plan != auto_plan:
+                            for _ in range(2):
+                                set_knobs(0, 0, 0)
+                                auto_runs.append(timed())
+                                set_knobs(best_plan[0], best_plan[1], best_plan[3])
+                                best_runs.append(timed())
+                    finally:
+                        set_knobs(0, 0, 0)
+                    auto_us, best_us = sorted(auto_runs)[len(auto_runs) // 2], sorted(best_runs)[len(best_runs) // 2]
+                    row = {"batch": batch, "c": c, "hw": hw, "dtype": "f16" if elt == 2 else "f32",
+                           "vectors_per_unit": c // 32 * hw * elt // 16, "units": batch * 32,
+                           "in_place": in_place, "auto": text(auto_plan), "auto_us": round(auto_us, 3),
+                           "best": text(best_plan), "best_us": round(best_us, 3),
+                           "auto_vs_best": round(auto_us / best_us, 3),
+                           "variants": {text(pl): round(us, 3) for pl, us in sorted(times.items())}}
+                    rows.append(row)
+                    if progress is not None:
+                        progress(row)
+                del case
+                torch.cuda.empty_cache()
+    return rows
+
+
+def sweep_summary(paths):
+    """Markdown summary of gn_plan_sweep rows read from JSON files (bench.py's output line or a
+    list of rows): per batch and call form the worst and median auto_vs_best, then every row whose
+    automatic plan is more than 3 % behind the fastest forced one."""
+    rows = []
+    for path in paths:
+        with open(path) as f:
+            for line in f:
+                line = line.strip()
+                if not line.startswith(("{", "[")):
+                    continue
+                data = json.loads(line)
+                rows += data["gn_plan_sweep"] if isinstance(data, dict) else data
+    out = ["| batch | call | rows | median auto / best | worst auto / best | worst row |", "|---:|---|---:|---:|---:|---|"]
+    for batch in sorted(set(r["batch"] for r in rows)):
+        for in_place in (True, False):
+            sel = [r for r in rows if r["batch"] == batch and r["in_place"] == in_place]
+            if not sel:
+                continue
+            ratios = sorted(r["auto_vs_best"] for r in sel)
+            worst = max(sel, key=lambda r: r["auto_vs_best"])
+            out.append("| %d | %s | %d | %.3f | %.3f | %d@%d %s: %s %.2f us, %s %.2f us |" % (
+                batch, "in place" if in_place else "apart", len(sel), ratios[len(ratios) // 2], ratios[-1],
+                worst["c"], worst["hw"], worst["dtype"], worst["auto"], worst["auto_us"], worst["best"], worst["best_us"]))
+    slow = [r for r in rows if r["auto_vs_best"] > 1.03]
+    out += ["", "Rows with the automatic plan more than 3 %% behind the fastest forced plan: %d of %d." % (len(slow), len(rows))]
+    if slow:
+        out += ["", "| batch | shape | dtype | call | automatic plan | us | fastest forced plan | us | ratio |",
+                "|---:|---|---|---|---|---:|---|---:|---:|"]
+        for r in sorted(slow, key=lambda r: -r["auto_vs_best"]):
+            out.append("| %d | %d@%d | %s | %s | %s | %.2f | %s | %.2f | %.3f |" % (
+                r["batch"], r["c"], r["hw"], r["dtype"], "in place" if r["in_place"] else "apart", r["auto"], r["auto_us"],
+                r["best"], r["best_us"], r["auto_vs_best"]))
+    return "\n".join(out)
+
+
+def trace_summary(trace_csv, bench_json):
+    """Markdown table: the rows of the `shapes` table of a profiled bench.py run next to the
+    device durations rocprofv3 --kernel-trace recorded for them.  The run's trace is cut at the
+    marker launches (TraceMarkers) whose labels the bench line carries in `trace_markers`; inside
+    a cut the kernel with the most dispatches is the measured one (the warm-up and the timed
+    replays), of which the median begin-to-end duration is reported per (kernel, grid, workgroup)."""
+    import csv
+    bench = None
+    with open(bench_json) as f:
+        for line in f:
+            if line.startswith("{"):
+                bench = json.loads(line)
+    labels = bench["trace_markers"]
+    disp = []
+    with open(trace_csv) as f:
+        for r in csv.DictReader(f):
+            disp.append((int(r["Start_Timestamp"]), int(r["End_Timestamp"]), r["Kernel_Name"],
+                         int(r["Grid_Size_X"]), int(r["Workgroup_Size_X"])))
+    disp.sort()
+    cuts, current = {}, None
+    for start, end, name, grid, wg in disp:
+        if "OpQuickGelu" in name and "__half" in name:
+            current = grid // 256 - 1
+            cuts[current] = []
+        elif current is not None:
+            cuts[current].append((name, grid, wg, end - start))
+
+    def short(name):
+        name = name.replace("msd::(anonymous namespace)::", "").replace("void ", "")
+        depth = 0
+        for i, ch in enumerate(name):
+            depth += ch == "<"
+            depth -= ch == ">"
+            if ch == "(" and depth == 0:
+                return name[:i]
+        return name
+
+    rows = bench["shapes"]
+    out = ["| config | kernel | shape | dtype | measurement | bytes | bench.py us (graph chain) | profiled kernel | grid x workgroup | dispatches | "
+           "median device us | GB/s at that | frac of 8 TB/s |", "|---|---|---|---|---|---:|---:|---|---|---:|---:|---:|---:|"]
+    for i, lab in enumerate(labels):
+        found = cuts.get(i, [])
+        if not found or lab["what"] == "memcpy_us":
+            continue
+        groups = {}
+        for name, grid, wg, dur in found:
+            groups.setdefault((name, grid, wg), []).append(dur)
+        (name, grid, wg), durs = max(groups.items(), key=lambda kv: len(kv[1]))
+        durs.sort()
+        med = durs[len(durs) // 2] / 1e3
+        row = rows[lab["row"]]
+        shape = " ".join("%s=%s" % kv for kv in row["shape"].items())
+        gbs = lab["bytes"] / med / 1e3
+        out.append("| %s | %s | %s | %s | %s | %d | %.2f | `%s` | %d x %d | %d | %.2f | %.0f | %.3f |" % (
+            row["config"], row["kernel"], shape, row["dtype"], lab["what"], lab["bytes"], row[lab["what"]], short(name),
+            grid // wg, wg, len(durs), med, gbs, gbs / HBM_PEAK_GBS))
+    return "\n".join(out)
 
 
 def fusion_table(torch, msd, dev, stream):
@@ -674,6 +952,7 @@ def large_batch_table(torch, msd, dev, stream):
     import ctypes
     vp = ctypes.c_void_p
     lib = msd.load_library()
+    rt = hip_runtime()
     F16 = msd.DTYPE_F16
     B = 32
     rows = []
@@ -721,6 +1000,10 @@ def large_batch_table(torch, msd, dev, stream):
         def copy_body():  # the same total bytes: read half, write half
             for x, y in zip(xs, ys):
                 assert lib.msd_copy(vp(x.data_ptr()), vp(y.data_ptr()), 2 * n_out, sp()) == 0
+
+        def memcpy_body():  # the same through the HIP runtime's own device-to-device copy
+            for x, y in zip(xs, ys):
+                assert rt.hipMemcpyDtoDAsync(vp(y.data_ptr()), vp(x.data_ptr()), 2 * n_out, sp()) == 0
         nbytes = 2 * (n_in + n_out)
         us = measure(body, copies)
         row = {"kernel": kind, "shape": p, "dtype": "f16", "bytes": nbytes, "us": round(us, 2),
@@ -729,6 +1012,9 @@ def large_batch_table(torch, msd, dev, stream):
             cus = measure(copy_body, copies)
             row["copy_us"] = round(cus, 2)
             row["pct_of_copy_rate"] = round(100 * cus / us, 1)
+            mus = measure(memcpy_body, copies)
+            row["memcpy_us"] = round(mus, 2)
+            row["pct_of_memcpy_rate"] = round(100 * mus / us, 1)
         if kind == "groupnorm_silu":
             row["plan"] = _gn_plan_text(msd, B, p["c"], p["hw"], 2)
         rows.append(row)
@@ -981,9 +1267,16 @@ def main():
     ap.add_argument("--mode", choices=["graph", "eager"], default="graph")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-kernel tables")
-    ap.add_argument("--tables", default="shapes,fusions,neighbours,large_batch",
-                    help="comma list of the per-kernel tables to measure (also: gn_split, the forced "
-                         "launch-plan sweep of GroupNorm)")
+    ap.add_argument("--tables", default="shapes,gn_split,fusions,neighbours,large_batch",
+                    help="comma list of the per-kernel tables to measure (also: gn_plan_sweep, the automatic "
+                         "GroupNorm launch plan against every forced one at --sweep-batches; minutes per batch)")
+    ap.add_argument("--sweep-batches", default="1,2,4,8,16,32", help="batches of the gn_plan_sweep table")
+    ap.add_argument("--sweep-summary", default=None, metavar="JSON[,JSON...]",
+                    help="no GPU: print the markdown summary of gn_plan_sweep rows in these bench.py outputs")
+    ap.add_argument("--trace-summary", default=None, metavar="KERNEL_TRACE_CSV",
+                    help="no GPU: print the `shapes` rows of --bench-json next to the device durations in this "
+                         "rocprofv3 --kernel-trace CSV of the same run")
+    ap.add_argument("--bench-json", default=None, help="the bench.py output (file) of the profiled run")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="for rocprofv3 --pmc runs: one 64 MiB device copy (known traffic) then three "
                          "eager steps; prints nothing")
@@ -992,6 +1285,12 @@ def main():
         print("bench.py measures one GPU: this path has no cross-GPU step and the build uses a single "
               "device; run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if args.sweep_summary:
+        print(sweep_summary(args.sweep_summary.split(",")))
+        return
+    if args.trace_summary:
+        print(trace_summary(args.trace_summary, args.bench_json))
+        return
 
     import ctypes
     import torch
@@ -1075,12 +1374,12 @@ def main():
 
     # One block per kernel family: algorithmic bytes per launch / live HIP-event time per launch
     # against the 8 TB/s peak, with the HBM traffic per launch that rocprofv3 --pmc FETCH_SIZE /
-    # WRITE_SIZE measured (profiles/traffic.json).  `roofline` is the single kernel with the
-    # largest total GPU time in the rocprofv3 kernel statistics of this workload,
+    # WRITE_SIZE measured (profiles/traffic.json).  The top level of `roofline` is the single kernel
+    # with the largest total GPU time in the rocprofv3 kernel statistics of this workload,
     # geglu_kernel<__half, 1>; the GroupNorm family as a whole takes more of the step and sits
-    # furthest below the roofline, which `roofline_families` shows.
+    # furthest below the roofline, which `roofline.families` shows.
     traffic = measured_traffic()
-    kernel_names = {"gn_silu": "gn_slice_kernel<__half, K, true>", "ln": "ln_team_kernel<__half, NW, VPL, TL>",
+    kernel_names = {"gn_silu": "gn_slice_kernel<__half, K, true, SHARED>", "ln": "ln_team_kernel<__half, NW, VPL, TL, EARLY>",
                     "geglu": "geglu_kernel<__half, 1>"}
     roofline_families = {}
     for kind, fam in families.items():
@@ -1091,6 +1390,7 @@ def main():
             "pct_of_step_time": round(100 * fam["us_total"] / (ms_per_step * 1e3), 1),
             "traffic": traffic.get(kind)}
     roofline = dict(roofline_families["geglu"])
+    roofline["families"] = roofline_families
 
     out = {
         "metric": "fused GroupNorm+SiLU/LayerNorm/GEGLU HBM GB/s over one SD UNet step (batch 2, fp16 storage)",
@@ -1104,7 +1404,6 @@ def main():
                    "copy_step_ms": round(copy_ms, 4), "pct_of_copy_step_rate": round(100 * copy_ms / ms_per_step, 1),
                    "ms_per_step_all_norms_out_of_place": round(apart_ms, 4)},
         "roofline": roofline,
-        "roofline_families": roofline_families,
         "kernel_families": families,
     }
     floor_us, graph_us = launch_floor_us(torch, msd, dev, stream)
@@ -1112,17 +1411,26 @@ def main():
     out["config"]["graph_launch_us"] = round(graph_us, 2)
     tables = set() if args.no_shapes else set(t for t in args.tables.split(",") if t)
     if "shapes" in tables:
-        out["shapes"] = shape_table(torch, msd, dev, stream)
+        markers = TraceMarkers(torch, msd, dev)
+        out["shapes"] = shape_table(torch, msd, dev, stream, floor_us, markers)
+        out["trace_markers"] = markers.labels
+    if "gn_split" in tables:
+        out["gn_split"] = gn_split_table(torch, msd, dev, stream)
     if "fusions" in tables:
         out["fusions"] = fusion_table(torch, msd, dev, stream)
     if "fusions" in tables:
         out["step_with_adds"] = step_with_adds(torch, msd, dev, stream)
     if "large_batch" in tables:
         out["large_batch"] = large_batch_table(torch, msd, dev, stream)
-    if "gn_split" in tables:
-        out["gn_split"] = gn_split_table(torch, msd, dev, stream)
     if "neighbours" in tables:
         out["neighbours"] = neighbour_table(torch, msd, dev, stream)
+    if "gn_plan_sweep" in tables:
+        def progress(row):  # a long table: one line per row on stderr keeps the run visibly alive
+            print("gn_plan_sweep batch %d %d@%d %s %s: auto %s %.2f us, best %s %.2f us" % (
+                row["batch"], row["c"], row["hw"], row["dtype"], "in place" if row["in_place"] else "apart",
+                row["auto"], row["auto_us"], row["best"], row["best_us"]), file=sys.stderr, flush=True)
+        out["gn_plan_sweep"] = gn_plan_sweep(torch, msd, dev, stream, [int(b) for b in args.sweep_batches.split(",") if b],
+                                             progress)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(step.bytes)
     else:

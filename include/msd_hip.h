@@ -50,8 +50,10 @@ const char *msd_error_string(int code);
  * (do not replay such a graph on a second stream while the first is busy with
  * GroupNorms).  Also looks up the device address of msd_groupnorm_noalloc's fixed
  * scratch on the current device.  hipStreamPerThread is refused (one handle, a
- * different stream in every thread).  No reference counterpart (the reference
- * allocates two temporaries per forward, M/nn/GroupNorm.cpp:95-103).
+ * different stream in every thread) - here and by msd_groupnorm, msd_chunk_add_groupnorm
+ * and msd_groupnorm_tokens for every shape, whether or not that launch would need the
+ * scratch; msd_groupnorm_noalloc, which has its own, takes it.  No reference counterpart
+ * (the reference allocates two temporaries per forward, M/nn/GroupNorm.cpp:95-103).
  */
 int msd_init(void *stream);
 
@@ -108,7 +110,9 @@ int msd_set_tuning(int knob, int value);
  * M/nn/ResBlock.cpp:222).  Requires channels % groups == 0.  When y lies apart from x
  * and there are fewer than 256 (sample, group) units, several workgroups share each unit
  * (msd_groupnorm_plan tells); the statistics are then summed in another order than for the
- * call in place, so the two results can differ in the last bit.
+ * call in place, so the two results can differ in the last bit.  A given call is
+ * reproducible bit for bit as long as msd_gn_fallbacks() stays 0: a workgroup that stopped
+ * waiting for a sibling sums that sibling's part in another order (same accuracy).
  */
 int msd_groupnorm(const void *x, void *y, const float *gamma, const float *beta,
                   size_t batch, size_t channels, size_t hw, size_t groups, float eps,
@@ -117,7 +121,8 @@ int msd_groupnorm(const void *x, void *y, const float *gamma, const float *beta,
 /*
  * msd_groupnorm for callers that cannot allocate (code under stream capture, tight serving
  * loops, harnesses that forbid hipMalloc): same arguments, same kernels, same result bit for
- * bit, but the workgroups' exchange area is a fixed 1 MiB array inside the library's code
+ * bit (while msd_gn_fallbacks() stays 0, see msd_groupnorm), but the workgroups' exchange
+ * area is a fixed 1 MiB array inside the library's code
  * object instead of a per-stream allocation, so the call never allocates or frees (its first
  * call on a device looks the array's address up; msd_init does that ahead of time).  Limit:
  * batch * groups <= 1024, otherwise MSD_ERR_SCRATCH_LIMIT.  Every stream of a device shares
@@ -181,9 +186,10 @@ int msd_layernorm(const void *x, void *y, const float *gamma, const float *beta,
  * c may alias a (every reference call site does) or b.
  *
  *   msd_chunk_add_groupnorm  = msd_chunkwise_add(x, chunk, tmp, ., hw) followed by
- *                      msd_groupnorm(tmp, y, ...), bit for bit, without the pass over tmp:
- *                      replaces M/nn/ResBlock.cpp:188-199 + 222-232 in one launch.
- *                      chunk is [batch, channels] in the activation storage type.
+ *                      msd_groupnorm(tmp, y, ...), bit for bit (while msd_gn_fallbacks() stays
+ *                      0, see msd_groupnorm), without the pass over tmp: replaces
+ *                      M/nn/ResBlock.cpp:188-199 + 222-232 in one launch.  chunk is
+ *                      [batch, channels] in the activation storage type and must not overlap y.
  *   msd_add_layernorm  = msd_elemwise_add(a, b, sum) followed by msd_layernorm(sum, y, ...), bit
  *                      for bit, in one launch; `sum` is written because the reference keeps it
  *                      as the next residual (M/nn/BasicTransformerBlock.cpp:126-136,149-158).
@@ -274,7 +280,8 @@ int msd_linear_rows(const void *x, const void *weight, const float *bias, void *
  * `silu(emb)` + `embed_linear->forward` pairs of one UNet step (M/nn/ResBlock.cpp:173-183),
  * which all read the one embedding that UNetModel::forward computes before its first block
  * (M/UNetModel.cpp:1107-1120), by one launch ahead of the blocks; each ys[i] equals what its
- * own msd_linear_rows call gives, bit for bit.  No ys[i] may overlap x.
+ * own msd_linear_rows call gives, bit for bit.  No ys[i] may overlap x, another ys[j], or
+ * any weights[j] / biases[j] (the problems run side by side); n and k are at most 2^28.
  */
 int msd_linear_rows_grouped(const void *x, const void *const *weights, const float *const *biases,
                             void *const *ys, const size_t *ns, size_t count, size_t m, size_t k,

@@ -256,7 +256,14 @@ static int groupnorm_entry(const void *x, const void *chunk, void *y, const floa
         count > (SIZE_MAX >> 3))
         return MSD_ERR_INVALID_VALUE;
     if (shifted_overlap(x, y, count * elt_bytes(dtype))) return MSD_ERR_INVALID_VALUE;
+    // the addend is read by every workgroup of its (sample, channel) while others already store
+    if (chunk != nullptr && ranges_overlap(chunk, batch * channels * elt_bytes(dtype), y, count * elt_bytes(dtype)))
+        return MSD_ERR_INVALID_VALUE;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    // Whether a launch needs the per-stream scratch depends on its shape; the rule does not:
+    // the one handle that names a different stream in every thread is refused for every call
+    // that may use that scratch (msd_groupnorm_noalloc, which has its own, takes it).
+    if (fixed == nullptr && s == hipStreamPerThread) return MSD_ERR_INVALID_VALUE;
     if (dtype == MSD_DTYPE_F32)
         return gn_dispatch<float>(x, chunk, y, gamma, beta, batch, channels, hw, groups, eps,
                                   fuse_silu != 0, fixed, s);
@@ -322,6 +329,7 @@ int msd_groupnorm_tokens(const void *x, void *y, const float *gamma, const float
         return MSD_ERR_INVALID_VALUE;
     if (ranges_overlap(x, count * elt_bytes(dtype), y, count * elt_bytes(dtype))) return MSD_ERR_INVALID_VALUE;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (s == hipStreamPerThread) return MSD_ERR_INVALID_VALUE;  // as for msd_groupnorm: may need the per-stream scratch
     if (dtype == MSD_DTYPE_F32)
         return gn_tokens_dispatch<float>(x, y, gamma, beta, batch, channels, hw, groups, eps, s);
     return gn_tokens_dispatch<__half>(x, y, gamma, beta, batch, channels, hw, groups, eps, s);
@@ -385,12 +393,10 @@ int msd_chunkwise_add(const void *a, const void *chunk, void *c, size_t n, size_
 int msd_geglu(const void *proj, void *out, size_t rows, size_t inner, int dtype, void *stream) {
     if (dtype != MSD_DTYPE_F32 && dtype != MSD_DTYPE_F16) return MSD_ERR_INVALID_VALUE;
     if (rows * inner != 0 && (!proj || !out)) return MSD_ERR_INVALID_VALUE;
-    {   // rows of proj and out have different strides: an overlapping out would be read after it was written
-        const size_t elt = dtype == MSD_DTYPE_F32 ? 4 : 2;
-        const uintptr_t p0 = reinterpret_cast<uintptr_t>(proj), o0 = reinterpret_cast<uintptr_t>(out);
-        const uintptr_t p1 = p0 + rows * 2 * inner * elt, o1 = o0 + rows * inner * elt;
-        if (rows * inner != 0 && o0 < p1 && p0 < o1) return MSD_ERR_INVALID_VALUE;
-    }
+    size_t count;
+    if (__builtin_mul_overflow(rows, inner, &count) || count > (SIZE_MAX >> 4)) return MSD_ERR_INVALID_VALUE;
+    // rows of proj and out have different strides: an overlapping out would be read after it was written
+    if (ranges_overlap(proj, 2 * count * elt_bytes(dtype), out, count * elt_bytes(dtype))) return MSD_ERR_INVALID_VALUE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == MSD_DTYPE_F32) return geglu_dispatch<float>(proj, out, rows, inner, s);
     return geglu_dispatch<__half>(proj, out, rows, inner, s);
@@ -483,12 +489,26 @@ int msd_linear_rows_grouped(const void *x, const void *const *weights, const flo
         return MSD_ERR_INVALID_VALUE;
     if (m > 8) return MSD_ERR_INVALID_VALUE;
     if (count != 0 && (!weights || !ys || !ns)) return MSD_ERR_INVALID_VALUE;
-    if (k > (SIZE_MAX >> 8)) return MSD_ERR_INVALID_VALUE;
+    constexpr size_t kMaxExtent = (size_t)1 << 28;  // keeps every byte count below far inside size_t
+    if (k > kMaxExtent) return MSD_ERR_INVALID_VALUE;
     for (size_t i = 0; i < count && m != 0; i++) {
         if (ns[i] == 0) continue;
-        if (!ys[i] || (k != 0 && (!x || !weights[i])) || ns[i] > (SIZE_MAX >> 8)) return MSD_ERR_INVALID_VALUE;
-        if (ranges_overlap(x, m * k * elt_bytes(dtype), ys[i], m * ns[i] * elt_bytes(dtype)))
-            return MSD_ERR_INVALID_VALUE;
+        if (!ys[i] || (k != 0 && (!x || !weights[i])) || ns[i] > kMaxExtent) return MSD_ERR_INVALID_VALUE;
+    }
+    // the problems run side by side in one launch: no output may lie in the shared rows or in
+    // any problem's output, weights or bias
+    const size_t elt = elt_bytes(dtype);
+    for (size_t i = 0; i < count && m != 0; i++) {
+        if (ns[i] == 0) continue;
+        const size_t ybytes = m * ns[i] * elt;
+        if (ranges_overlap(x, m * k * elt, ys[i], ybytes)) return MSD_ERR_INVALID_VALUE;
+        for (size_t j = 0; j < count; j++) {
+            if (ns[j] == 0) continue;
+            if (j != i && ranges_overlap(ys[j], m * ns[j] * elt, ys[i], ybytes)) return MSD_ERR_INVALID_VALUE;
+            if (k != 0 && ranges_overlap(weights[j], ns[j] * k * elt, ys[i], ybytes)) return MSD_ERR_INVALID_VALUE;
+            if (biases && biases[j] && ranges_overlap(biases[j], ns[j] * sizeof(float), ys[i], ybytes))
+                return MSD_ERR_INVALID_VALUE;
+        }
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == MSD_DTYPE_F32)

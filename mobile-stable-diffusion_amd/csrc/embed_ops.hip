@@ -354,9 +354,9 @@ void softmax_flat_launch(const T *x, T *y, uint32_t blocks, uint32_t cols, int s
     const size_t lds = (size_t)RB * cols * sizeof(T);  // a whole number of 16-byte vectors: RB is a multiple of 8
     constexpr int kFew = (80 + TEAM - 1) / TEAM, kMany = kSmFlatMaxCols / TEAM;
     if (cols <= 80)
-        hipLaunchKernelGGL((softmax_flat_kernel<T, RB, kFew, TEAM>), dim3(blocks), dim3(RB * TEAM), lds, stream, x, y, cols, stable);
+        launch((softmax_flat_kernel<T, RB, kFew, TEAM>), dim3(blocks), dim3(RB * TEAM), lds, stream, x, y, cols, stable);
     else
-        hipLaunchKernelGGL((softmax_flat_kernel<T, RB, kMany, TEAM>), dim3(blocks), dim3(RB * TEAM), lds, stream, x, y, cols, stable);
+        launch((softmax_flat_kernel<T, RB, kMany, TEAM>), dim3(blocks), dim3(RB * TEAM), lds, stream, x, y, cols, stable);
 }
 
 // ---------------------------------------------------------------------------
@@ -408,10 +408,10 @@ void linear_launch(const T *x, const T *w, const float *bias, T *y, uint32_t m, 
                    int act_in, int act_out, hipStream_t stream) {
     constexpr int EPV = Store<T>::EPV;
     if (act_in)  // two columns per wavefront share the activated x
-        hipLaunchKernelGGL((linear_rows_kernel<T, M, 2>), dim3((n + 1) / 2), dim3(kWave), 0, stream, x, w, bias,
+        launch((linear_rows_kernel<T, M, 2>), dim3((n + 1) / 2), dim3(kWave), 0, stream, x, w, bias,
                            y, m, n, k / EPV, act_in, act_out);
     else
-        hipLaunchKernelGGL((linear_rows_kernel<T, M, 1>), dim3(n), dim3(kWave), 0, stream, x, w, bias, y, m, n,
+        launch((linear_rows_kernel<T, M, 1>), dim3(n), dim3(kWave), 0, stream, x, w, bias, y, m, n,
                            k / EPV, act_in, act_out);
 }
 
@@ -422,7 +422,7 @@ void softmax_team_launch(const T *x, T *y, uint32_t rows, uint32_t row_vecs, int
     // workgroups: 3 % faster at 65536 x 4096; the shorter ones keep 256 lanes
     constexpr uint32_t threads = (TL == kWave && VPL >= 8) ? kWave : kSmThreads;
     constexpr uint32_t rows_per_block = (threads / kWave) * (kWave / TL);
-    hipLaunchKernelGGL((softmax_team_kernel<T, VPL, TL>), dim3((rows + rows_per_block - 1) / rows_per_block),
+    launch((softmax_team_kernel<T, VPL, TL>), dim3((rows + rows_per_block - 1) / rows_per_block),
                        dim3(threads), 0, stream, x, y, rows, row_vecs, stable);
 }
 
@@ -448,7 +448,7 @@ int linear_rows_dispatch(const void *xv, const void *wv, const float *bias, void
         }
     } else {
         const uint32_t blocks = (uint32_t)((n + kLinWaves - 1) / kLinWaves);
-        hipLaunchKernelGGL((linear_rows_generic_kernel<T>), dim3(blocks), dim3(kLinThreads), 0, stream, x,
+        launch((linear_rows_generic_kernel<T>), dim3(blocks), dim3(kLinThreads), 0, stream, x,
                            w, bias, y, (uint32_t)m, (uint32_t)n, (uint32_t)k, act_in, act_out);
     }
     return launch_status();
@@ -462,16 +462,16 @@ void linear_grouped_launch(const T *x, const LinearGroup &g, uint32_t m, uint32_
     constexpr int EPV = Store<T>::EPV;
     const uint32_t blocks = g.first_block[g.count];
     if (cpw == 4 && k / EPV > 128 && k / EPV <= 192)  // three pieces per lane cover the row (k = 1280: 3 % faster)
-        hipLaunchKernelGGL((linear_rows_grouped_kernel<__half, (M <= 2 ? M : 1), 4, 3>), dim3(blocks), dim3(kWave), 0,
+        launch((linear_rows_grouped_kernel<__half, (M <= 2 ? M : 1), 4, 3>), dim3(blocks), dim3(kWave), 0,
                            stream, reinterpret_cast<const __half *>(x), g, m, k / EPV, act_in, act_out);
     else if (cpw == 4)  // (only 2-byte elements and up to two rows: see the dispatch)
-        hipLaunchKernelGGL((linear_rows_grouped_kernel<__half, (M <= 2 ? M : 1), 4>), dim3(blocks), dim3(kWave), 0,
+        launch((linear_rows_grouped_kernel<__half, (M <= 2 ? M : 1), 4>), dim3(blocks), dim3(kWave), 0,
                            stream, reinterpret_cast<const __half *>(x), g, m, k / EPV, act_in, act_out);
     else if (cpw == 2)
-        hipLaunchKernelGGL((linear_rows_grouped_kernel<T, M, 2>), dim3(blocks), dim3(kWave), 0, stream, x, g, m,
+        launch((linear_rows_grouped_kernel<T, M, 2>), dim3(blocks), dim3(kWave), 0, stream, x, g, m,
                            k / EPV, act_in, act_out);
     else
-        hipLaunchKernelGGL((linear_rows_grouped_kernel<T, M, 1>), dim3(blocks), dim3(kWave), 0, stream, x, g, m,
+        launch((linear_rows_grouped_kernel<T, M, 1>), dim3(blocks), dim3(kWave), 0, stream, x, g, m,
                            k / EPV, act_in, act_out);
 }
 
@@ -601,11 +601,11 @@ int softmax_dispatch(const void *xv, void *yv, size_t rows, size_t cols, int sta
     const uint32_t r_left = (uint32_t)rows;
     const dim3 grid((uint32_t)((rows + waves_per_block - 1) / waves_per_block));
     if (cols <= 2 * kWave)
-        hipLaunchKernelGGL((softmax_short_kernel<T, 2>), grid, dim3(kSmThreads), 0, stream, x, y, r_left, c, stable);
+        launch((softmax_short_kernel<T, 2>), grid, dim3(kSmThreads), 0, stream, x, y, r_left, c, stable);
     else if (cols <= 8 * kWave)
-        hipLaunchKernelGGL((softmax_short_kernel<T, 8>), grid, dim3(kSmThreads), 0, stream, x, y, r_left, c, stable);
+        launch((softmax_short_kernel<T, 8>), grid, dim3(kSmThreads), 0, stream, x, y, r_left, c, stable);
     else
-        hipLaunchKernelGGL((softmax_generic_kernel<T>), grid, dim3(kSmThreads), 0, stream, x, y, r_left, c, stable);
+        launch((softmax_generic_kernel<T>), grid, dim3(kSmThreads), 0, stream, x, y, r_left, c, stable);
     return launch_status();
 }
 
@@ -620,7 +620,7 @@ int ddim_update_dispatch(const void *xv, const void *ev, void *yv, size_t n, flo
     c.sqrt_aprev = sqrtf(a_prev);
     const int vectors = aligned16(xv) && aligned16(ev) && aligned16(yv);
     const size_t want = (n / Store<T>::EPV + kDdimThreads) / kDdimThreads;
-    hipLaunchKernelGGL((ddim_update_kernel<T>), dim3((uint32_t)(want < 4096 ? want : 4096)),
+    launch((ddim_update_kernel<T>), dim3((uint32_t)(want < 4096 ? want : 4096)),
                        dim3(kDdimThreads), 0, stream, static_cast<const T *>(xv),
                        static_cast<const T *>(ev), static_cast<T *>(yv), n, vectors, c);
     return launch_status();

@@ -109,12 +109,15 @@ __device__ __forceinline__ void gn_exchange(const GnScratch &scratch, const GnPa
         if (tid < p.split) {
             unsigned long long wm, wq;
             uint32_t polls = 0;
+            // A slice never gives up on its own words: they arrive without anybody's help, and
+            // having read them back is what lets it store output (see below).
+            const uint32_t limit = tid == slice ? 0xFFFFFFFFu : p.spin_limit;
             do {
                 wm = __hip_atomic_load(slot_mean + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 wq = __hip_atomic_load(slot_m2 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 ok = (uint32_t)(wm >> 32) == tag && (uint32_t)(wq >> 32) == tag;
                 if (!ok) __builtin_amdgcn_s_sleep(1);
-            } while (!ok && ++polls < p.spin_limit);
+            } while (!ok && ++polls < limit);
             m_l = __uint_as_float((uint32_t)wm);
             q_l = __uint_as_float((uint32_t)wq);
             const uint32_t b = tid * p.vec_per_slice;
@@ -123,9 +126,12 @@ __device__ __forceinline__ void gn_exchange(const GnScratch &scratch, const GnPa
         }
         // Slices that have not published (not dispatched yet, or starved): this wavefront
         // computes their (mean, M2) from their part of the input, two passes.  A slice stores
-        // output only after it has seen every word of its unit, this slice's included, so what
-        // is read here is still input unless the sibling published in the meantime - then its
-        // words are there when they are read again after the passes, and they win.
+        // output only after it has read back every word of its unit from the memory side, its
+        // own included, so what is read here is still input unless the sibling published in the
+        // meantime - then its words are at the memory side before its first output store
+        // leaves, and they win when they are read again after the passes.  That second read
+        // must not start before the passes' loads have returned: the wait below stops the
+        // memory pipeline, and as a compiler barrier the compiler, from moving it ahead.
         unsigned long long missing = __builtin_amdgcn_ballot_w64(!ok);
         if (missing != 0) {  // uniform over the wavefront
             while (missing != 0) {
@@ -152,6 +158,7 @@ __device__ __forceinline__ void gn_exchange(const GnScratch &scratch, const GnPa
                     }
                 }
                 const float m2_s = wave_sum(q);
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 if (tid == s) {
                     const unsigned long long wm =
                         __hip_atomic_load(slot_mean + s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -850,16 +857,16 @@ void gn_launch_k(bool silu, bool shared, uint32_t blocks, uint32_t threads, hipS
     if (K <= kGnSharedMaxK && shared) {
         constexpr int KS = K <= kGnSharedMaxK ? K : 1;  // (larger K never get here: no such instances)
         if (silu)
-            hipLaunchKernelGGL((gn_slice_kernel<T, KS, true, true>), dim3(blocks), dim3(threads), 0, stream, x,
+            launch((gn_slice_kernel<T, KS, true, true>), dim3(blocks), dim3(threads), 0, stream, x,
                                chunk, y, gamma, beta, sc, p);
         else
-            hipLaunchKernelGGL((gn_slice_kernel<T, KS, false, true>), dim3(blocks), dim3(threads), 0, stream,
+            launch((gn_slice_kernel<T, KS, false, true>), dim3(blocks), dim3(threads), 0, stream,
                                x, chunk, y, gamma, beta, sc, p);
     } else if (silu) {
-        hipLaunchKernelGGL((gn_slice_kernel<T, K, true, false>), dim3(blocks), dim3(threads), 0, stream, x,
+        launch((gn_slice_kernel<T, K, true, false>), dim3(blocks), dim3(threads), 0, stream, x,
                            chunk, y, gamma, beta, sc, p);
     } else {
-        hipLaunchKernelGGL((gn_slice_kernel<T, K, false, false>), dim3(blocks), dim3(threads), 0, stream,
+        launch((gn_slice_kernel<T, K, false, false>), dim3(blocks), dim3(threads), 0, stream,
                            x, chunk, y, gamma, beta, sc, p);
     }
 }
@@ -868,7 +875,7 @@ template <typename T>
 int gn_generic(bool silu, const T *x, const T *chunk, T *y, const float *gamma, const float *beta,
                size_t units, size_t unit_size, size_t hw, size_t groups, size_t cpg, float eps,
                hipStream_t stream) {
-    hipLaunchKernelGGL((silu ? gn_generic_kernel<T, true> : gn_generic_kernel<T, false>),
+    launch((silu ? gn_generic_kernel<T, true> : gn_generic_kernel<T, false>),
                        dim3((uint32_t)units), dim3(kGenericThreads), 0, stream, x, chunk, y, gamma, beta,
                        (uint32_t)unit_size, (uint32_t)hw, (uint32_t)groups, (uint32_t)cpg, eps);
     return launch_status();
@@ -1130,10 +1137,10 @@ void gn_tokens_launch(bool shared, uint32_t blocks, uint32_t threads, size_t lds
                       const GnTokParams &q) {
     if (K <= kGnSharedMaxK && shared) {
         constexpr int KS = K <= kGnSharedMaxK ? K : 1;  // (no instances with several writers beyond that)
-        hipLaunchKernelGGL((gn_tokens_kernel<T, KS, true>), dim3(blocks), dim3(threads), lds_bytes, stream, x, y,
+        launch((gn_tokens_kernel<T, KS, true>), dim3(blocks), dim3(threads), lds_bytes, stream, x, y,
                            gamma, beta, sc, q);
     } else {
-        hipLaunchKernelGGL((gn_tokens_kernel<T, K, false>), dim3(blocks), dim3(threads), lds_bytes, stream, x, y,
+        launch((gn_tokens_kernel<T, K, false>), dim3(blocks), dim3(threads), lds_bytes, stream, x, y,
                            gamma, beta, sc, q);
     }
 }
@@ -1154,7 +1161,7 @@ int gn_tokens_dispatch(const void *xv, void *yv, const float *gamma, const float
     if (units == 0 || unit_size == 0) return MSD_OK;
     if (units > 0x7FFFFFFFull || unit_size > 0x7FFFFFFFull) return MSD_ERR_INVALID_VALUE;
     auto generic = [&]() {
-        hipLaunchKernelGGL((gn_tokens_generic_kernel<T>), dim3((uint32_t)units), dim3(kGenericThreads), 0,
+        launch((gn_tokens_generic_kernel<T>), dim3((uint32_t)units), dim3(kGenericThreads), 0,
                            stream, x, y, gamma, beta, (uint32_t)unit_size, (uint32_t)hw, (uint32_t)groups,
                            (uint32_t)cpg, eps);
         return launch_status();

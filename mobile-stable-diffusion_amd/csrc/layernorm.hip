@@ -1,9 +1,12 @@
 // LayerNorm for gfx950: a row is owned by a team of TL adjacent lanes of one
 // wavefront (TL = 4..64), VPL 16-byte vectors per lane, so a wavefront covers
 // 64/TL consecutive rows and every load instruction fetches whole 128-byte lines.
-// Mean and M2 are computed from registers in two passes (exact centred variance),
-// reduced across the team with DPP; gamma / beta are fetched while the row data is
-// in flight.  One HBM read and one HBM write per element.
+// Mean and M2 come from one pass of sum and sum of squares over the packed registers, reduced
+// across the team with DPP; a wavefront in which some row's mean is large against its spread
+// (|mean| > 2 sigma, or a constant row) takes a second, centred pass over the registers, so the
+// variance is as accurate as a two-pass one either way.  gamma / beta are fetched while the row
+// data is in flight (small launches) or staged in LDS once per workgroup.  One HBM read and one
+// HBM write per element.
 #include "msd_device.h"
 #include "msd_internal.h"
 
@@ -276,10 +279,10 @@ void ln_launch(const T *x, const T *res, T *sum, T *y, const float *gamma, const
     const uint32_t rows_per_block = (kWave / TL) * (threads / kWave);
     const uint32_t blocks = (rows + rows_per_block - 1) / rows_per_block;
     if (early)
-        hipLaunchKernelGGL((ln_team_kernel<T, NW, VPL, TL, true>), dim3(blocks), dim3(threads), 0, stream, x,
+        launch((ln_team_kernel<T, NW, VPL, TL, true>), dim3(blocks), dim3(threads), 0, stream, x,
                            res, sum, y, gamma, beta, rows, eps, inv_dim);
     else
-        hipLaunchKernelGGL((ln_team_kernel<T, NW, VPL, TL, false>), dim3(blocks), dim3(threads),
+        launch((ln_team_kernel<T, NW, VPL, TL, false>), dim3(blocks), dim3(threads),
                            2 * sizeof(float) * VPL * TL * (NW * 4 / sizeof(T)), stream, x, res, sum, y, gamma, beta,
                            rows, eps, inv_dim);
 }
@@ -361,7 +364,7 @@ int ln_dispatch(const void *xv, const void *resv, void *sumv, void *yv, const fl
     }
     if (!done) {
         const uint32_t rows_per_block = kLnThreads / kWave;
-        hipLaunchKernelGGL((ln_generic_kernel<T>),
+        launch((ln_generic_kernel<T>),
                            dim3((uint32_t)((rows + rows_per_block - 1) / rows_per_block)),
                            dim3(kLnThreads), 0, stream, x, res, sum, y, gamma, beta, (uint32_t)rows,
                            (uint32_t)dim, eps);

@@ -5,13 +5,43 @@
 #include <atomic>
 #include <stddef.h>
 #include <stdint.h>
+#include <tuple>
+#include <utility>
 
 #include "../../include/msd_hip.h"
 
 namespace msd {
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
-inline int launch_status() { return (int)hipGetLastError(); }
+
+// Kernel launches go through hipLaunchKernel, which returns the status of that launch itself;
+// nothing reads or clears the thread's "last error" of the HIP runtime, so an error that an
+// unrelated earlier call of the application left there is neither reported as ours nor lost.
+// launch() keeps the first failure of the calling thread's launches until launch_status()
+// returns it (and forgets it): a dispatcher launches, then returns launch_status().
+inline thread_local hipError_t t_launch_error = hipSuccess;
+
+template <typename... KArgs, typename... Args, size_t... I>
+inline hipError_t launch_with(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t lds, hipStream_t stream,
+                              std::index_sequence<I...>, Args &&...args) {
+    std::tuple<KArgs...> values(static_cast<KArgs>(std::forward<Args>(args))...);
+    void *pointers[sizeof...(KArgs) + 1] = {const_cast<void *>(static_cast<const void *>(&std::get<I>(values)))..., nullptr};
+    return hipLaunchKernel(reinterpret_cast<const void *>(kernel), grid, block, pointers, lds, stream);
+}
+
+template <typename... KArgs, typename... Args>
+inline void launch(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t lds, hipStream_t stream, Args &&...args) {
+    static_assert(sizeof...(KArgs) == sizeof...(Args), "one argument per kernel parameter");
+    const hipError_t err = launch_with(kernel, grid, block, lds, stream, std::index_sequence_for<KArgs...>{},
+                                       std::forward<Args>(args)...);
+    if (err != hipSuccess && t_launch_error == hipSuccess) t_launch_error = err;
+}
+
+inline int launch_status() {
+    const hipError_t err = t_launch_error;
+    t_launch_error = hipSuccess;
+    return (int)err;
+}
 
 // ---- GroupNorm scratch: what workgroups sharing one (sample, group) exchange ----
 constexpr uint32_t kGnMaxSplit = 64;    // workgroups per unit (one wavefront reads all slots)

@@ -322,15 +322,15 @@ int geglu_dispatch(const void *pv, void *ov, size_t rows, size_t inner, hipStrea
         const uint32_t ov = (uint32_t)out_vecs;
         auto blocks = [&](int u) { return (uint32_t)((out_vecs + kGegluThreads * u - 1) / (kGegluThreads * u)); };
         if (unroll == 1)
-            hipLaunchKernelGGL((geglu_kernel<T, 1>), dim3(blocks(1)), dim3(kGegluThreads), 0, stream, proj, out, ov, fd);
+            launch((geglu_kernel<T, 1>), dim3(blocks(1)), dim3(kGegluThreads), 0, stream, proj, out, ov, fd);
         else if (unroll == 2)
-            hipLaunchKernelGGL((geglu_kernel<T, 2>), dim3(blocks(2)), dim3(kGegluThreads), 0, stream, proj, out, ov, fd);
+            launch((geglu_kernel<T, 2>), dim3(blocks(2)), dim3(kGegluThreads), 0, stream, proj, out, ov, fd);
         else
-            hipLaunchKernelGGL((geglu_kernel<T, 4>), dim3(blocks(4)), dim3(kGegluThreads), 0, stream, proj, out, ov, fd);
+            launch((geglu_kernel<T, 4>), dim3(blocks(4)), dim3(kGegluThreads), 0, stream, proj, out, ov, fd);
     } else {
         const size_t n = rows * inner;
         const size_t want = (n + kStreamThreads - 1) / kStreamThreads;
-        hipLaunchKernelGGL((geglu_generic_kernel<T>), dim3((uint32_t)(want < 65536 ? want : 65536)),
+        launch((geglu_generic_kernel<T>), dim3((uint32_t)(want < 65536 ? want : 65536)),
                            dim3(kStreamThreads), 0, stream, proj, out, rows, inner);
     }
     return launch_status();
@@ -350,17 +350,17 @@ int act_launch(const void *xv, void *yv, size_t n, hipStream_t stream) {
         const int unroll = tune_vectors ? tune_vectors : kStreamUnroll;
         const uint32_t blocks = vecs ? stream_blocks(vecs, unroll) : 1u;
         if (unroll == 4)
-            hipLaunchKernelGGL((act_kernel<T, OP, 4>), dim3(blocks), dim3(kStreamThreads), 0, stream, x, y,
+            launch((act_kernel<T, OP, 4>), dim3(blocks), dim3(kStreamThreads), 0, stream, x, y,
                                (uint32_t)vecs, n);
         else if (unroll == 2)
-            hipLaunchKernelGGL((act_kernel<T, OP, 2>), dim3(blocks), dim3(kStreamThreads), 0, stream, x, y,
+            launch((act_kernel<T, OP, 2>), dim3(blocks), dim3(kStreamThreads), 0, stream, x, y,
                                (uint32_t)vecs, n);
         else
-            hipLaunchKernelGGL((act_kernel<T, OP, 1>), dim3(blocks), dim3(kStreamThreads), 0, stream, x, y,
+            launch((act_kernel<T, OP, 1>), dim3(blocks), dim3(kStreamThreads), 0, stream, x, y,
                                (uint32_t)vecs, n);
     } else {
         const size_t want = (n + kStreamThreads - 1) / kStreamThreads;
-        hipLaunchKernelGGL((act_generic_kernel<T, OP>),
+        launch((act_generic_kernel<T, OP>),
                            dim3((uint32_t)(want < 65536 ? want : 65536)), dim3(kStreamThreads), 0,
                            stream, x, y, n);
     }
@@ -384,11 +384,11 @@ int add_dispatch(const void *av, const void *bv, void *cv, size_t n, size_t chun
         const uint32_t vecs = (uint32_t)(n / EPV);
         FastDiv fd = make_fast_div((uint32_t)(chunk_size / EPV));
         if (chunk_size == 0) fd.d = 0;
-        hipLaunchKernelGGL((add_kernel<T>), dim3((vecs + kStreamThreads - 1) / kStreamThreads),
+        launch((add_kernel<T>), dim3((vecs + kStreamThreads - 1) / kStreamThreads),
                            dim3(kStreamThreads), 0, stream, a, b, c, vecs, fd);
     } else {
         const size_t want = (n + kStreamThreads - 1) / kStreamThreads;
-        hipLaunchKernelGGL((add_generic_kernel<T>), dim3((uint32_t)(want < 65536 ? want : 65536)),
+        launch((add_generic_kernel<T>), dim3((uint32_t)(want < 65536 ? want : 65536)),
                            dim3(kStreamThreads), 0, stream, a, b, c, n, chunk_size);
     }
     return launch_status();
@@ -415,19 +415,19 @@ int permute_021_dispatch(const void *srcv, void *dstv, size_t isize, size_t jsiz
     // copy takes 29.1; the other way round nothing changes).
     const bool jfast = jsize < ksize;
     if (words && jfast && tiles.x <= 65535) {
-        hipLaunchKernelGGL((permute_021_words_kernel<(int)sizeof(T), true>), dim3(tiles.y, tiles.x, tiles.z), dim3(256), 0,
+        launch((permute_021_words_kernel<(int)sizeof(T), true>), dim3(tiles.y, tiles.x, tiles.z), dim3(256), 0,
                            stream, srcv, dstv, (uint32_t)jsize, (uint32_t)ksize);
     } else if (words) {
-        hipLaunchKernelGGL((permute_021_words_kernel<(int)sizeof(T), false>), tiles, dim3(256), 0, stream, srcv, dstv,
+        launch((permute_021_words_kernel<(int)sizeof(T), false>), tiles, dim3(256), 0, stream, srcv, dstv,
                            (uint32_t)jsize, (uint32_t)ksize);
     } else if (tiled) {
-        hipLaunchKernelGGL((permute_021_kernel<T>),
+        launch((permute_021_kernel<T>),
                            dim3((uint32_t)((ksize + kTile - 1) / kTile), (uint32_t)((jsize + kTile - 1) / kTile),
                                 (uint32_t)isize),
                            dim3(256), 0, stream, src, dst, (uint32_t)jsize, (uint32_t)ksize);
     } else {
         const size_t want = (isize * jsize * ksize + kStreamThreads - 1) / kStreamThreads;
-        hipLaunchKernelGGL((permute_021_generic_kernel<T>), dim3((uint32_t)(want < 65536 ? want : 65536)),
+        launch((permute_021_generic_kernel<T>), dim3((uint32_t)(want < 65536 ? want : 65536)),
                            dim3(kStreamThreads), 0, stream, src, dst, isize, jsize, ksize);
     }
     return launch_status();
@@ -450,7 +450,7 @@ int temb_dispatch(const int64_t *timesteps, void *out, size_t batch, size_t dim,
     const uint32_t half = (uint32_t)(dim / 2);
     const uint32_t blocks = (uint32_t)((batch * half + 255) / 256);
     const float neg_log_period = -logf(max_period);  // host float log, as in the replaced host loop
-    hipLaunchKernelGGL((timestep_embedding_kernel<T>), dim3(blocks), dim3(256), 0, stream, timesteps,
+    launch((timestep_embedding_kernel<T>), dim3(blocks), dim3(256), 0, stream, timesteps,
                        static_cast<T *>(out), (uint32_t)batch, half, neg_log_period);
     return launch_status();
 }

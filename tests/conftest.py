@@ -33,6 +33,38 @@ def pytest_sessionfinish(session, exitstatus):
             json.dump(merged, f, indent=1, sort_keys=True)
 
 
+def _product():
+    return importlib.import_module("mobile-stable-diffusion_amd")
+
+
+@pytest.fixture(autouse=True)
+def _gn_fallbacks_start_at_zero(request):
+    """Results that are promised bit for bit hold while no GroupNorm workgroup gave up waiting
+    for a sibling (msd_gn_fallbacks() == 0).  Every GPU test starts with the counter at zero, so
+    that a failing test's report (below) can say whether that happened during the test."""
+    if request.node.get_closest_marker("gpu") is not None:
+        try:
+            import torch
+            if torch.cuda.is_available():
+                _product().gn_fallbacks(reset=True)
+        except Exception:
+            pass
+    yield
+
+
+@pytest.hookimpl(hookwrapper=True)
+def pytest_runtest_makereport(item, call):
+    outcome = yield
+    report = outcome.get_result()
+    if report.when == "call" and report.failed and item.get_closest_marker("gpu") is not None:
+        try:
+            count = _product().gn_fallbacks()
+            report.sections.append(("msd_gn_fallbacks", "workgroups that computed a sibling's statistics themselves "
+                                    "during this test (current stream and the fixed scratch): %d" % count))
+        except Exception as exc:  # the device may be what failed
+            report.sections.append(("msd_gn_fallbacks", "not readable: %r" % (exc,)))
+
+
 @pytest.fixture(scope="session")
 def msd():
     """The product package (ctypes access to the HIP library); raises if it is not built."""

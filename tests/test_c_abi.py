@@ -120,6 +120,11 @@ def test_shifted_overlaps_are_refused_before_any_launch(msd):
     gn = lambda x, y: lib.msd_groupnorm(p(x), p(y), p(w), p(w), 2, 64, 16, 32, f(1e-5), 1, 1, None)
     assert gn(base, base + 2048) == 1 and gn(base + 4094, base) == 1
     assert lib.msd_chunk_add_groupnorm(p(base), p(w), p(base + 64), p(w), p(w), 2, 64, 16, 32, f(1e-5), 1, 1, None) == 1
+    # the per-(sample, channel) addend ([2, 64] fp16 = 256 bytes) inside the output, in place and apart
+    far_y = base + (1 << 16)
+    chunk_gn = lambda chunk, y: lib.msd_chunk_add_groupnorm(p(base), p(chunk), p(y), p(w), p(w), 2, 64, 16, 32,
+                                                            f(1e-5), 1, 1, None)
+    assert chunk_gn(base + 1024, base) == 1 and chunk_gn(far_y + 4094, far_y) == 1 and chunk_gn(far_y - 2, far_y) == 1
     tok = lambda x, y: lib.msd_groupnorm_tokens(p(x), p(y), p(w), p(w), 2, 64, 16, 32, f(1e-6), 1, None)
     assert tok(base, base) == 1 and tok(base, base + 4094) == 1 and tok(base + 2, base) == 1
     # [8, 64] fp32 = 2048 bytes
@@ -146,6 +151,18 @@ def test_shifted_overlaps_are_refused_before_any_launch(msd):
     ws = (ctypes.c_void_p * 2)(w, w)
     ns = (ctypes.c_size_t * 2)(4, 4)
     assert lib.msd_linear_rows_grouped(p(base), ws, None, ys, ns, 2, 2, 8, 0, 0, 0, None) == 1
+    # the problems of a grouped launch run side by side: outputs ([2, 4] fp32 = 32 bytes) may not
+    # overlap each other, nor any problem's weights ([4, 8] fp32 = 128 bytes) or bias (16 bytes)
+    def grouped(y0, y1, w0=w, w1=w + 4096, b0=None, b1=None):
+        ys_ = (ctypes.c_void_p * 2)(y0, y1)
+        ws_ = (ctypes.c_void_p * 2)(w0, w1)
+        bs_ = None if b0 is None and b1 is None else (ctypes.c_void_p * 2)(b0, b1)
+        return lib.msd_linear_rows_grouped(p(base), ws_, bs_, ys_, ns, 2, 2, 8, 0, 0, 0, None)
+    assert grouped(far, far) == 1 and grouped(far, far + 28) == 1                 # output in output
+    assert grouped(far, far + 64, w1=far - 64) == 1                               # output 0 in the weights of problem 1
+    assert grouped(far, far + 64, w0=far + 32) == 1                               # output 1 in the weights of problem 0
+    assert grouped(far, far + 64, b0=far + 4096, b1=far + 72) == 1                # output 1 in a bias
+    assert lib.msd_linear_rows_grouped(p(base), ws, None, ys, ns, 2, 2, (1 << 28) + 8, 0, 0, 0, None) == 1  # k too long
     assert lib.msd_softmax(p(base), p(base + 2), 4, 77, 0, 1, None) == 1
     upd = lambda x, e, y: lib.msd_ddim_update(p(x), p(e), p(y), 64, f(0.5), f(0.6), f(0.7), 0, None)
     assert upd(base, far, base + 4) == 1 and upd(base, far, far + 252) == 1
@@ -154,6 +171,24 @@ def test_shifted_overlaps_are_refused_before_any_launch(msd):
     assert lib.msd_silu(p(base), p(far), huge, 0, None) == 1
     assert lib.msd_permute_0_2_1(p(base), p(far), 1 << 31, 1 << 31, 8, 1, None) == 1
     assert lib.msd_groupnorm(p(base), p(far), p(w), p(w), 1 << 40, 32, 1 << 30, 32, f(1e-5), 0, 0, None) == 1
+    assert lib.msd_geglu(p(base), p(far), 1 << 40, 1 << 30, 1, None) == 1
+    assert lib.msd_geglu(p(base), p(far), 1 << 31, 1 << 29, 0, None) == 1         # 2 * rows * inner * 4 bytes: 2^63
+
+
+def test_stream_per_thread_is_refused_for_every_groupnorm_that_may_use_the_stream_scratch(msd):
+    """hipStreamPerThread names a different stream in every thread, so it cannot key the
+    per-stream scratch: the calls that may need that scratch refuse it whatever the shape (a
+    small unit that would not be cut as well as a large one), before anything is launched."""
+    lib = msd.load_library()
+    p, f = ctypes.c_void_p, ctypes.c_float
+    per_thread = p(2)  # the value of hipStreamPerThread
+    x, y, w = 1 << 20, 1 << 22, 1 << 24
+    for channels, hw in ((64, 16), (320, 4096)):
+        assert lib.msd_groupnorm(p(x), p(y), p(w), p(w), 2, channels, hw, 32, f(1e-5), 1, 1, per_thread) == 1
+        assert lib.msd_groupnorm(p(x), p(x), p(w), p(w), 2, channels, hw, 32, f(1e-5), 1, 1, per_thread) == 1
+        assert lib.msd_chunk_add_groupnorm(p(x), p(w), p(y), p(w), p(w), 2, channels, hw, 32, f(1e-5), 1, 1,
+                                           per_thread) == 1
+        assert lib.msd_groupnorm_tokens(p(x), p(y), p(w), p(w), 2, channels, hw, 32, f(1e-6), 1, per_thread) == 1
 
 
 def test_missing_library_fails_loudly(msd):

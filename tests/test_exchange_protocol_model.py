@@ -5,18 +5,20 @@ What the kernel does per slice, and what the model replays one memory operation 
 
   1. read the unit's launch count `epoch` (once, at kernel start); tag = epoch + 1
   2. publish (tag, mean) and (tag, M2) of its own part as two separate 64-bit words
-  3. lane l polls slice l's two words until both carry the tag, at most `spin_limit` times;
-     a sibling that has not published by then is computed from the sibling's part of the INPUT
-     (two passes), after which its words are read once more and win if they have arrived
+  3. lane l polls slice l's two words until both carry the tag, at most `spin_limit` times -
+     without limit for the slice's OWN words, which arrive without anybody's help; a sibling
+     that has not published by then is computed from the sibling's part of the INPUT (two
+     passes, all of whose loads have returned before the next step), after which its words are
+     read once more and win if they have arrived
   4. merge all slices (Chan), then fetch_add(done) (its old value is used in step 6)
   5. only now store the output over its own part (the call may be in place)
   6. the slice whose fetch_add returned split - 1 stores done = 0, epoch = tag
 
 All of it is relaxed atomics: stores become visible to the other slices after arbitrary delays
-and in any order across addresses.  Two things the protocol leans on are modelled as facts of
-the machine: a kernel's stores are all visible when the next launch on the stream starts, and a
-slice's output stores (issued after a full poll round trip) do not become visible before its
-own two words, which it issued earlier on the same path.
+and in any order across addresses.  One thing the protocol leans on is modelled as a fact of
+the machine: a kernel's stores are all visible when the next launch on the stream starts.  That
+a slice's output never becomes visible before its own two words is not assumed: the slice
+issues its output stores only after it has read both words back.
 
 Checked over many random schedules, several consecutive launches per unit and changing split
 factors: a word of an earlier launch is never accepted, every slice ends up with the statistics
@@ -71,16 +73,13 @@ class Launch:
             self.overwritten[index] = True
 
     def committable(self):
-        """Indices of pending stores that may become visible now: the oldest one per address,
-        and a slice's output only after its own two words."""
+        """Indices of pending stores that may become visible now: the oldest one per address."""
         seen, ok = set(), []
         for i, (s, kind, index, value) in enumerate(self.pending):
             key = (kind, index)
             if key in seen:
                 continue
             seen.add(key)
-            if kind == "output" and any(p[0] == s and p[1] in ("mean", "m2") for p in self.pending[:i]):
-                continue
             ok.append(i)
         return ok
 
@@ -107,7 +106,7 @@ class Launch:
                 waiting.remove(l)
                 continue
             polls[l] += 1
-            if polls[l] >= self.spin_limit:   # give up on slice l: compute it from its input
+            if l != s and polls[l] >= self.spin_limit:   # give up on sibling l: compute it from its input
                 clean = not self.overwritten[l]
                 yield                         # (the two passes over the sibling's input)
                 clean = clean and not self.overwritten[l]
