@@ -546,7 +546,9 @@ def gn_plan_sweep(torch, msd, dev, stream, batches, progress=None):
     2 / 4 / 8 writers per whole unit x the same workgroup sizes).  A forced setting counts only if
     msd_groupnorm_plan confirms that the launch follows it; identical plans are timed once.  The
     automatic plan and the fastest forced one are then timed twice more, alternating, and
-    `auto_vs_best` is the ratio of the medians: above 1.03 the planner picked a slow variant."""
+    `auto_vs_best` is the ratio of the medians: above 1.03 the planner picked a slow variant.  `rule`
+    / `rule_vs_best`: the same for the planning rule alone, with the table of measured plans (which the
+    automatic plan consults first) switched off."""
     lib = msd.load_library()
     knobs = (msd.TUNE_GN_SPLIT, msd.TUNE_GN_THREADS, msd.TUNE_GN_WRITERS)
 
@@ -573,6 +575,12 @@ def gn_plan_sweep(torch, msd, dev, stream, batches, progress=None):
                         set_knobs(0, 0, 0)
                         auto_plan = msd.groupnorm_plan(batch, c, hw, 32, code, in_place=in_place)
                         times = {auto_plan: timed()}
+                        # the rule alone (the table of measured plans switched off)
+                        assert lib.msd_set_tuning(msd.TUNE_GN_PLAN_RULE_ONLY, 1) == 0
+                        rule_plan = msd.groupnorm_plan(batch, c, hw, 32, code, in_place=in_place)
+                        if rule_plan not in times:
+                            times[rule_plan] = timed()
+                        assert lib.msd_set_tuning(msd.TUNE_GN_PLAN_RULE_ONLY, 0) == 0
                         for writers in ((1,) if in_place else (1, 2, 4, 8)):
                             for split in ((1, 2, 4, 8) if writers == 1 else (1,)):
                                 for threads in SWEEP_THREADS:
@@ -592,12 +600,15 @@ def gn_plan_sweep(torch, msd, dev, stream, batches, progress=None):
                                 best_runs.append(timed())
                     finally:
                         set_knobs(0, 0, 0)
+                        lib.msd_set_tuning(msd.TUNE_GN_PLAN_RULE_ONLY, 0)
                     auto_us, best_us = sorted(auto_runs)[len(auto_runs) // 2], sorted(best_runs)[len(best_runs) // 2]
                     row = {"batch": batch, "c": c, "hw": hw, "dtype": "f16" if elt == 2 else "f32",
                            "vectors_per_unit": c // 32 * hw * elt // 16, "units": batch * 32,
                            "in_place": in_place, "auto": text(auto_plan), "auto_us": round(auto_us, 3),
                            "best": text(best_plan), "best_us": round(best_us, 3),
                            "auto_vs_best": round(auto_us / best_us, 3),
+                           "rule": text(rule_plan), "rule_us": round(times[rule_plan], 3),
+                           "rule_vs_best": round(times[rule_plan] / min(best_us, times[rule_plan]), 3),
                            "variants": {text(pl): round(us, 3) for pl, us in sorted(times.items())}}
                     rows.append(row)
                     if progress is not None:
@@ -620,7 +631,8 @@ def sweep_summary(paths):
                     continue
                 data = json.loads(line)
                 rows += data["gn_plan_sweep"] if isinstance(data, dict) else data
-    out = ["| batch | call | rows | median auto / best | worst auto / best | worst row |", "|---:|---|---:|---:|---:|---|"]
+    out = ["| batch | call | rows | median auto / best | worst auto / best | worst row | rule alone: median | worst | rows > 1.03 |",
+           "|---:|---|---:|---:|---:|---|---:|---:|---:|"]
     for batch in sorted(set(r["batch"] for r in rows)):
         for in_place in (True, False):
             sel = [r for r in rows if r["batch"] == batch and r["in_place"] == in_place]
@@ -628,9 +640,11 @@ def sweep_summary(paths):
                 continue
             ratios = sorted(r["auto_vs_best"] for r in sel)
             worst = max(sel, key=lambda r: r["auto_vs_best"])
-            out.append("| %d | %s | %d | %.3f | %.3f | %d@%d %s: %s %.2f us, %s %.2f us |" % (
+            rule = sorted(r.get("rule_vs_best", float("nan")) for r in sel)
+            out.append("| %d | %s | %d | %.3f | %.3f | %d@%d %s: %s %.2f us, %s %.2f us | %.3f | %.3f | %d |" % (
                 batch, "in place" if in_place else "apart", len(sel), ratios[len(ratios) // 2], ratios[-1],
-                worst["c"], worst["hw"], worst["dtype"], worst["auto"], worst["auto_us"], worst["best"], worst["best_us"]))
+                worst["c"], worst["hw"], worst["dtype"], worst["auto"], worst["auto_us"], worst["best"], worst["best_us"],
+                rule[len(rule) // 2], rule[-1], sum(1 for v in rule if v > 1.03)))
     slow = [r for r in rows if r["auto_vs_best"] > 1.03]
     out += ["", "Rows with the automatic plan more than 3 %% behind the fastest forced plan: %d of %d." % (len(slow), len(rows))]
     if slow:

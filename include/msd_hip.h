@@ -98,6 +98,11 @@ int msd_gn_fallbacks(void *stream, unsigned int *count, int reset);
                                      that sibling's statistics itself (tests set 1 to exercise that path) */
 #define MSD_TUNE_GN_WRITERS 8     /* workgroups that share one whole (sample, group), each storing a part
                                      of it: 1 (never), 2, 4, 8 or 16 (wherever the launch allows it) */
+#define MSD_TUNE_DEVICE_CUS 9     /* plan GroupNorm launches for a chip of this many compute units instead of
+                                     asking the current device (tests; 0: ask) */
+#define MSD_TUNE_DEVICE_XCDS 10   /* ... and of this many XCDs, each with an L2 of its own (0: ask) */
+#define MSD_TUNE_GN_PLAN_RULE_ONLY 11 /* 1: ignore the table of measured GroupNorm plans, plan by the rule alone
+                                     (benchmark sweeps measure the rule with it) */
 int msd_set_tuning(int knob, int value);
 
 /*

@@ -18,7 +18,8 @@ LIB_NN_PATH = os.path.join(CSRC_DIR, "libmsd_nn.so")
 DTYPE_F32 = 0
 DTYPE_F16 = 1
 TUNE_GN_SPLIT, TUNE_GN_THREADS, TUNE_LN_CHUNK, TUNE_LN_THREADS, TUNE_GEGLU_VECTORS, TUNE_ACT_VECTORS, \
-    TUNE_SOFTMAX_ROWS, TUNE_GN_SPIN_LIMIT, TUNE_GN_WRITERS = range(9)
+    TUNE_SOFTMAX_ROWS, TUNE_GN_SPIN_LIMIT, TUNE_GN_WRITERS, TUNE_DEVICE_CUS, TUNE_DEVICE_XCDS, \
+    TUNE_GN_PLAN_RULE_ONLY = range(12)
 ERR_SCRATCH_LIMIT = -2
 
 # every symbol include/msd_hip.h declares

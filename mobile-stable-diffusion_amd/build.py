@@ -40,7 +40,7 @@ def _run(cmd):
     return out
 
 
-HIP_SOURCES = ["api.hip", "groupnorm.hip", "layernorm.hip", "stream_ops.hip", "embed_ops.hip"]
+HIP_SOURCES = ["api.hip", "gn_plan.hip", "groupnorm.hip", "layernorm.hip", "stream_ops.hip", "embed_ops.hip"]
 
 
 def build_hip():
@@ -52,7 +52,7 @@ def build_hip():
         src, obj = pair
         return _run([HIPCC] + DEVICE_FLAGS + ["-c", "-o", obj, os.path.join(CSRC, src)])
 
-    with ThreadPoolExecutor(max_workers=5) as pool:
+    with ThreadPoolExecutor(max_workers=6) as pool:
         list(pool.map(compile_one, zip(HIP_SOURCES, objs)))
     _run([HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-Wno-unused-command-line-argument",
           "-o", LIB_HIP] + objs)

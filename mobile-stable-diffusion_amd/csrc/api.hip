@@ -228,6 +228,18 @@ int msd_set_tuning(int knob, int value) {
             if (value && ((value & (value - 1)) != 0 || value > 16)) return MSD_ERR_INVALID_VALUE;
             g_tuning.gn_writers = value;
             return MSD_OK;
+        case MSD_TUNE_DEVICE_CUS:
+            if (value > 4096) return MSD_ERR_INVALID_VALUE;
+            g_tuning.device_cus = value;
+            return MSD_OK;
+        case MSD_TUNE_DEVICE_XCDS:
+            if (value > 64) return MSD_ERR_INVALID_VALUE;
+            g_tuning.device_xcds = value;
+            return MSD_OK;
+        case MSD_TUNE_GN_PLAN_RULE_ONLY:
+            if (value > 1) return MSD_ERR_INVALID_VALUE;
+            g_tuning.gn_plan_rule_only = value;
+            return MSD_OK;
         default:
             return MSD_ERR_INVALID_VALUE;
     }

@@ -38,14 +38,8 @@ namespace msd {
 
 namespace {
 
-constexpr int kGnMaxThreads = 1024;
-constexpr int kGnMaxK = 20;        // vectors per lane; the largest only for slices it fits exactly
-constexpr int kGnMaxRaggedK = 16;  // the largest with code for a ragged slice
 constexpr uint32_t kGnSpinLimit = 2048;  // default poll limit: about half a microsecond per poll
 constexpr int kGenericThreads = 256;
-constexpr size_t kChipCus = 256;  // compute units of an MI355X
-constexpr int kGnPrefetchAffineK = 6;       // vectors per lane up to which gamma / beta are kept in registers
-constexpr uint32_t kGnLdsChannels = 1024;  // channels per group the LDS copy of gamma / beta has room for
 
 struct GnParams {
     uint32_t vec_per_unit;   // 16-byte vectors per unit
@@ -63,7 +57,8 @@ struct GnParams {
     uint32_t writers;        // power of two
     uint32_t writers_shift;  // log2(writers)
     uint32_t part_vecs;      // vectors per part, a multiple of 64 (a wavefront is inside one part or outside)
-    uint32_t same_xcd;       // the writers of a unit have block ids 8 apart: one XCD, one L2 (units % 8 == 0)
+    uint32_t xcd_shift;      // the writers of a unit have block ids (1 << xcd_shift) apart: with that many XCDs they
+                             // share one XCD and its L2 (units in whole rows of that many); 0: adjacent ids
 };
 
 // Sum over the workgroup (blockDim.x / 64 wavefronts); one barrier.
@@ -491,10 +486,9 @@ __global__ __launch_bounds__(kGnMaxThreads, (K <= (sizeof(T) == 2 ? 5 : 4) ? 8 :
     __shared__ float2 aff[K <= kGnPrefetchAffineK ? 1 : kGnLdsChannels];  // (gamma, beta) of the group's channels
     uint32_t unit, slice, part;
     if (SHARED) {  // whole units, `writers` workgroups each
-        const uint32_t j = p.same_xcd ? blockIdx.x >> 3 : blockIdx.x;
+        const uint32_t j = blockIdx.x >> p.xcd_shift;
         part = j & (p.writers - 1);
-        unit = j >> p.writers_shift;
-        if (p.same_xcd) unit = (unit << 3) + (blockIdx.x & 7);
+        unit = ((j >> p.writers_shift) << p.xcd_shift) + (blockIdx.x & ((1u << p.xcd_shift) - 1u));
         slice = 0;
     } else {
         unit = blockIdx.x >> p.split_shift;
@@ -571,7 +565,8 @@ struct GnTokParams {
 // SHARED: `writers` workgroups per whole unit (output apart from the input by construction).  Each
 // loads and reduces the whole unit, enumerated part by part (a part = all channels over a range of
 // positions, what a slice is above), and normalises, transposes and stores its own part; nothing
-// is exchanged.  The writers of a unit have block ids 8 apart (one XCD: their loads meet in its L2).
+// is exchanged.  The writers of a unit have block ids one XCD count apart (one XCD: their loads meet in
+// its L2).
 template <typename T, int K, bool SHARED>
 __global__ __launch_bounds__(kGnMaxThreads) void gn_tokens_kernel(
     const T *__restrict__ x, T *__restrict__ y, const float *__restrict__ gamma,
@@ -592,10 +587,9 @@ __global__ __launch_bounds__(kGnMaxThreads) void gn_tokens_kernel(
     // the slices of a unit stay adjacent
     uint32_t unit, slice;  // SHARED: `slice` is the part this workgroup stores
     if (SHARED) {
-        const uint32_t j = p.same_xcd ? blockIdx.x >> 3 : blockIdx.x;
+        const uint32_t j = blockIdx.x >> p.xcd_shift;
         slice = j & (p.writers - 1);
-        unit = j >> p.writers_shift;
-        if (p.same_xcd) unit = (unit << 3) + (blockIdx.x & 7);
+        unit = ((j >> p.writers_shift) << p.xcd_shift) + (blockIdx.x & ((1u << p.xcd_shift) - 1u));
     } else {
         const uint32_t group = fast_div(blockIdx.x, q.combos);
         const uint32_t combo = blockIdx.x - group * q.combos.d;
@@ -724,131 +718,15 @@ __global__ __launch_bounds__(kGenericThreads) void gn_tokens_generic_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// Host: launch plan
+// Host: launches (the plan comes from gn_plan.hip)
 // ---------------------------------------------------------------------------
-const int kKValues[] = {1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 20};
-
-inline int round_up_k(uint32_t k) {
-    for (int v : kKValues)
-        if ((uint32_t)v >= k) return v;
-    return 0;
+// log2 of the distance between the block ids of a unit's writers: the XCD count when the
+// workgroups of a launch are dealt to a power-of-two number of XCDs in turn and the units come
+// in whole rows of that many (the writers then share an XCD), else 0 (adjacent ids).
+inline uint32_t gn_xcd_shift(const GnChip &chip, bool shared, size_t units) {
+    if (!shared || chip.xcds <= 1 || (chip.xcds & (chip.xcds - 1)) != 0 || units % chip.xcds != 0) return 0;
+    return (uint32_t)__builtin_ctz(chip.xcds);
 }
-
-struct GnPlan {
-    uint32_t split;
-    uint32_t threads;
-    int k;  // 0 = does not fit
-};
-
-// K for a slice of `vecs` vectors on `threads` lanes, 0 if there is none.  The largest K has
-// no code for a ragged slice: it takes equal slices that it fits exactly.
-int k_for(uint32_t vecs, uint32_t threads, uint32_t max_k, bool equal_slices) {
-    const int k = round_up_k((vecs + threads - 1) / threads);
-    if (k == 0 || (uint32_t)k > max_k) return 0;
-    if (k == kGnMaxK && !(equal_slices && vecs == (uint32_t)k * threads)) return 0;
-    return k;
-}
-
-// 640 ... 1024 lanes that hold a slice of `vecs` vectors as exactly 1 ... max_fit_k vectors per
-// lane (nothing masked), 0 if there is no such size.  Measured against the next power-of-two
-// size with a masked tail, 2-byte elements: 1280-vector slices 5.97 us on 640 lanes against 6.20
-// on 1024, 1920-vector units 4.24 us on 960 lanes against 4.35 on 512 (three or four vectors per
-// lane gain nothing there).  4-byte elements gain up to four vectors per lane: 3840-vector slices
-// 12.28 us on 960 x 4 against 12.55 on 512 x 8, 2560-vector slices 7.12 on 640 x 4 against 7.23
-// on 1024 x 3.
-uint32_t exact_fit_threads(uint32_t vecs, uint32_t max_fit_k) {
-    for (uint32_t k = 1; k <= max_fit_k; k++)
-        for (uint32_t t = kGnMaxThreads; t >= 640; t -= kWave)
-            if (vecs == k * t) return t;
-    return 0;
-}
-
-// Threads and K for a slice of `vecs` vectors.  Measured on MI355X over every UNet shape
-// (workgroups of 256 ... 1024 lanes in steps of 64, 1 - 8 slices per unit): for a launch of
-// few workgroups 512 lanes finish soonest whenever the slice is at most 5 vectors per lane,
-// larger slices want 1024 lanes, and a small whole unit runs best with exactly one vector per
-// lane.  The tail of a slice that does not fill K * threads is masked.
-GnPlan plan_slice(uint32_t vecs, uint32_t split, uint32_t force_threads, uint32_t max_k, bool equal_slices,
-                  size_t blocks = 0, size_t elt = 2, bool shared = false) {
-    GnPlan pl{split, 0, 0};
-    if (force_threads && k_for(vecs, force_threads, max_k, equal_slices) != 0) {
-        pl.threads = force_threads;
-    } else if (blocks >= 2 * kChipCus && vecs >= 256) {
-        // Two or more workgroups per CU (large batches): throughput counts, not one workgroup's
-        // latency, and small workgroups that each hold many vectors per lane do best - more of
-        // them share a CU, in different phases (load / statistics / store), and a barrier joins
-        // four wavefronts, not sixteen.  Measured at batch 32 (1024 units), fp16, us per launch
-        // with 256 / 512 / 1024 lanes: 5120-vector units 30.1 / 33.6 / 31.8, 2560: 14.8 / 15.5 /
-        // 18.4, 1920: 12.0 / 13.1 / 15.4, 3840: 23.3 / 24.9 / 24.9; fp32 5120: 29.5 / 29.8 / 33.9.
-        // Batch 16 (512 units), 5120: 14.95 / 15.2 / 15.2; batch 12 is where 256 lanes lose
-        // (13.9 / 13.3 / 13.4) and the rules below take over.
-        // Exactly two or three workgroups per CU that are slices of cut units (4-byte elements at
-        // batch 2 - 8) still want large workgroups: 3840-vector slices 12.28 us on 960 x 4 against
-        // 12.55 on 512 x 8, 5120-vector slices 14.6 us on 512 x 10 against 14.8 on 640 x 8.
-        const bool cut_few = split > 1 && blocks < 4 * kChipCus;
-        if (cut_few) {
-            // ... as long as a CU has room for all of its workgroups at once (a SIMD holds eight
-            // wavefronts and takes a quarter of each workgroup's, rounded up): 768 slices of 3840
-            // vectors take 16.5 us on 512 x 8 and 18.7 on 960 x 4, of which only two fit a CU
-            const uint32_t exact = exact_fit_threads(vecs, elt == 2 ? 2 : 4);
-            if (exact != 0 && (blocks + kChipCus - 1) / kChipCus <= 8 / ((exact + 255) / 256)) pl.threads = exact;
-        }
-        // 1024 and more slices of cut units, more than 384 units: the smallest workgroup that holds a slice in at most
-        // five vectors per lane (against 256 lanes with eight or ten: 1920-vector slices 64.5 us on
-        // 384 x 5 against 66.9, 2560-vector slices 83.2 on 512 x 5 against 87.3, 3840-vector slices
-        // 122 on 768 x 5 against 127, batch 24, 4-byte elements)
-        if (split > 1 && !cut_few && blocks / split > 384)
-            for (uint32_t t = 384; t <= kGnMaxThreads && pl.threads == 0; t += 128) {
-                const int k = k_for(vecs, t, max_k, equal_slices);
-                if (k != 0 && k <= 5) pl.threads = t;
-            }
-        for (uint32_t t : {256u, 512u, 768u, 1024u}) {
-            if (pl.threads != 0) break;
-            if ((cut_few && t == 256u) || k_for(vecs, t, max_k, equal_slices) == 0) continue;
-            // (short slices: at least ten wavefronts per CU - 512 units of 2560 vectors 8.54 us
-            // on 512 x 5 against 8.98 on 256 x 10, of 3840 vectors 11.9 on 512 x 8 against 12.7)
-            if (vecs <= 4096 && (size_t)t * blocks < 10 * kWave * kChipCus && t < kGnMaxThreads) continue;
-            pl.threads = t;
-        }
-        if (pl.threads == 0) pl.threads = kGnMaxThreads;
-    } else if (shared && vecs <= 2560) {
-        // Whole units that several writers share (every workgroup reduces all of the unit, a
-        // part of its wavefronts does the epilogue): fewer lanes with more vectors each than
-        // for one writer.  Measured at batch 2 with four writers, fp16: 640-vector units 2.79 us
-        // on 384 x 2 against 2.89 on 640 x 1, 1920 vectors 3.36 on 512 x 4 against 3.56 on
-        // 960 x 2; fp32 2560 vectors 3.76 on 640 x 4 against 3.89 on 512 x 5.
-        pl.threads = vecs == 2560 ? 640u : vecs > 704 ? 512u : vecs >= 256 ? 384u : ((vecs + kWave - 1) / kWave) * kWave;
-    } else if (uint32_t exact = (split == 1 && vecs == (elt == 2 ? 1280u : 2560u))
-                                    ? 0u
-                                    : exact_fit_threads(vecs, elt == 2 ? 2 : 4)) {
-        // (a whole unit of 10240 elements is the exception.  2-byte elements: 3.55 us on 512
-        // lanes with a masked tail against 3.62 us on 640 x 2; 4-byte elements: 512 x 5 is an
-        // exact fit itself, 3.98 us against 4.08 on 640 x 4)
-        pl.threads = exact;
-    } else if (!shared && split == 1 && vecs > 5120 && vecs % 640 == 0 && vecs / 10 >= 640 && vecs / 10 <= kGnMaxThreads &&
-               max_k >= 10) {
-        // long whole units that are exactly ten vectors per lane on 640 ... 1024 lanes (7680-vector
-        // units of 4-byte elements: 8.05 us on 768 x 10 against 8.44 on 1024 x 8 with a masked tail)
-        pl.threads = vecs / 10;
-    } else if (!shared && elt == 4 && split == 1 && vecs == 5120 && blocks >= 160) {
-        // whole 5120-vector units of 4-byte elements from batch 5 on: 512 x 10 (batch 7 / 8: 7.38 /
-        // 8.12 us against 7.79 / 8.49 on 1024 x 5; the same at batch 2 - 5)
-        pl.threads = 512;
-    } else if (vecs > 512u * 5u || (split > 1 && vecs >= 960))  // slices of a cut unit: 2 - 3 % faster
-        pl.threads = kGnMaxThreads;
-    else if (split == 1 && vecs >= 256 && vecs <= 704 && vecs % kWave == 0)
-        pl.threads = vecs;  // one vector per lane, nothing masked: 3 % faster for the 8 x 8 maps
-    else if (vecs >= 256)
-        pl.threads = 512;
-    else
-        pl.threads = ((vecs + kWave - 1) / kWave) * kWave;
-    pl.k = k_for(vecs, pl.threads, max_k, equal_slices);
-    return pl;
-}
-
-// Kernels with several writers per unit exist up to this many vectors per lane (units of up
-// to 10240 vectors on 1024 lanes).
-constexpr int kGnSharedMaxK = 10;
 
 template <typename T, int K>
 void gn_launch_k(bool silu, bool shared, uint32_t blocks, uint32_t threads, hipStream_t stream, const T *x,
@@ -882,178 +760,6 @@ int gn_generic(bool silu, const T *x, const T *chunk, T *y, const float *gamma, 
 }
 
 }  // namespace
-
-// Writers per whole unit when the launch may share units (1: it does not).  A unit's time is
-// its load, its statistics and the epilogue of SiLU and stores, one behind the other on one
-// CU; with w workgroups per unit, each loading and reducing all of it (the copies meet in the
-// L2 of the XCD they share) and finishing a w-th of it, the epilogue and the stores shrink to
-// a w-th while nothing is exchanged.  Best where it gives the chip about one workgroup per CU
-// (measured on every UNet shape, fp16 / fp32, us per launch against the usual plan; 64 units:
-// 2560 vectors 4.76 -> 4.34 (2 writers) -> 4.06 (4) -> 5.07 (8); 5120 vectors, otherwise cut
-// in four with an exchange, 6.00 -> 5.33 (4); 32 units: 2560 vectors 4.59 -> 3.59 (8); 128
-// units: 4.70 (2) against 5.09 and 5.62 (4); 256 units and more: always slower).  Past 5120
-// vectors of 2-byte elements (10240 of 4-byte ones, 5120 with eight writers) the repeated
-// loads cost more than the shorter epilogue gains (7680 vectors, 64 units: 6.71 against 6.56
-// cut in four).
-uint32_t gn_auto_writers(size_t elt, size_t units, size_t vec_per_unit) {
-    // The writers of a unit must run on one XCD (block ids 8 apart: workgroups are dealt to the
-    // XCDs in turn), which needs the units in whole rows of 8; on adjacent blocks, that is on
-    // different XCDs, every copy comes from memory: 5.28 us for the 4.76 above.
-    if (units % 8 != 0) return 1;
-    uint32_t w = 1;
-    while (w < 8 && units * w * 2 <= kChipCus) w *= 2;
-    const size_t limit = (elt == 2 || w >= 8) ? 5120 : 10240;
-    return vec_per_unit <= limit ? w : 1;
-}
-
-// What a GroupNorm launch looks like for a shape: split == 0 means the general kernel (one
-// workgroup per unit, any alignment); otherwise `split` workgroups of `threads` lanes per unit,
-// each holding its slice as `k` vectors per lane.  `elt` = bytes per element, `max_units` = units
-// the exchange scratch has room for.  `writers` > 1 (only where `may_share`: the output does
-// not overlap the input) means whole units with that many workgroups each, every one loading and
-// reducing the whole unit and storing its part of it.  Reads the tuning knobs.
-GnDecision gn_decide(size_t elt, size_t batch, size_t channels, size_t hw, size_t groups, bool aligned,
-                     size_t max_units, bool may_share) {
-    GnDecision d{0, 0, 0, 0, 1};
-    const size_t epv = 16 / elt;
-    const int tune_split = g_tuning.gn_split.load(std::memory_order_relaxed);
-    const int tune_threads = g_tuning.gn_threads.load(std::memory_order_relaxed);
-    const size_t cpg = channels / groups;
-    const size_t unit_size = cpg * hw;
-    const size_t units = batch * groups;
-    // (the register kernel addresses a unit with 32-bit byte offsets)
-    if (!aligned || hw % epv != 0 || unit_size * elt >= (1ull << 32)) return d;
-
-    const size_t vec_per_unit = unit_size / epv;
-    constexpr uint32_t kMaxK = kGnMaxK;
-
-    // ---- several writers per whole unit
-    const int tune_writers = g_tuning.gn_writers.load(std::memory_order_relaxed);
-    if (may_share && tune_split <= 1 && tune_writers != 1 && vec_per_unit <= (size_t)kGnMaxThreads * kGnSharedMaxK) {
-        uint32_t writers = tune_writers > 1 ? (uint32_t)tune_writers : gn_auto_writers(elt, units, vec_per_unit);
-        while (writers > 1 && vec_per_unit < (size_t)writers * kWave) writers /= 2;  // a part is at least a wavefront's vectors
-        if (units * writers > 0x7FFFFFFFull) writers = 1;                            // (the grid is units * writers blocks)
-        if (writers > 1) {
-            uint32_t force = 0;
-            if (tune_threads >= kWave && tune_threads <= kGnMaxThreads && tune_threads % kWave == 0 &&
-                (size_t)tune_threads * kGnSharedMaxK >= vec_per_unit)
-                force = (uint32_t)tune_threads;
-            const GnPlan pl = plan_slice((uint32_t)vec_per_unit, 1, force, kGnSharedMaxK, true, units * writers, elt, true);
-            if (pl.k != 0 && !(pl.k > kGnPrefetchAffineK && cpg > kGnLdsChannels)) {
-                d.split = 1;
-                d.threads = pl.threads;
-                d.k = (uint32_t)pl.k;
-                d.vec_per_slice = (uint32_t)vec_per_unit;
-                d.writers = writers;
-                return d;
-            }
-        }
-    }
-
-    const size_t slice_cap = (size_t)kGnMaxThreads * kGnMaxRaggedK;  // vectors one workgroup can hold
-    // smallest power-of-two split whose slices fit in registers
-    uint32_t split = 1;
-    while ((size_t)split * slice_cap < vec_per_unit && split <= kGnMaxSplit) split *= 2;
-    const bool can_split = units <= max_units;
-    if (split > kGnMaxSplit || (split > 1 && !can_split)) return d;
-    if (tune_split > 0) {
-        uint32_t forced = (uint32_t)tune_split;
-        if (forced > split && can_split && (forced & (forced - 1)) == 0 && forced <= kGnMaxSplit &&
-            vec_per_unit >= (size_t)forced * kWave)
-            split = forced;
-    } else if (can_split) {
-        // A workgroup's time grows with its slice (one CU loads, reduces and normalises it) while
-        // the exchange between the slices of a unit costs 1.3 - 1.9 us (two round trips through
-        // the memory-side coherence point), so units up to 24 Ki elements stay whole and larger
-        // ones are cut in two or four; eight when that still leaves most of the chip idle.
-        // With 256 or more units every CU has one of its own and cutting only adds the exchange
-        // (batch 8, 320 channels at 64x64: 9.0 us whole against 10.5 us in two).
-        uint32_t want = 1;
-        if (elt == 2) {
-            if (unit_size > 24576) {
-                // (up to 32 Ki elements two slices are enough from 64 units on: 960 channels at
-                // 32 x 32, batch 2, 5.40 us in two against 5.63 us in four; batch 1 4.86 in four
-                // against 5.03 in two)
-                // (96 units, batch 3: 320 channels at 64 x 64 6.44 us in two against 6.74 in four)
-                want = units >= 256 ? 1
-                       : (units >= 128 || (unit_size <= 32768 && units >= 64) || (unit_size <= 61440 && units >= 96)) ? 2
-                                                                                                                      : 4;
-                // (batch 1: 960 channels at 64 x 64 7.08 us in eight against 7.16 in four, 640
-                // channels 6.56 against 6.12)
-                if (units * 4 < 192 && unit_size > 98304) want = 8;
-                // 160 ... 224 units (batch 5 - 7): two slices would give some CUs two 1024-lane
-                // workgroups and others one, so units stay whole (one workgroup on most CUs) or,
-                // the long ones, go in four on 512 lanes (three small workgroups per CU).  Batch 5 /
-                // 6 / 7, us whole against in two: 320 channels at 64 x 64 7.67 / 8.02 / 8.49 against
-                // 8.57 / 8.95 / 9.27, 960 at 32 x 32 6.45 / 6.75 / 7.00 against 7.28 / 7.64 / 7.86;
-                // in four against in two: 640 at 64 x 64 12.3 / 13.3 / - against 13.7 / 14.3, 960 at
-                // 64 x 64 17.6 / 18.7 / - against 19.9 / 20.9 (batch 7: whole, 20.7 against 22.0).
-                if (units > 128 && units < 256) want = (units >= 224 || unit_size <= 61440) ? 1 : 4;
-            }
-        } else {
-            // 4-byte elements, half the arithmetic per vector: whole up to 5120 vectors (4096 when
-            // the units alone fill less than a quarter of the chip), then halved until the slices
-            // are at most 5120 vectors or the launch would pass two workgroups per CU; a launch
-            // of fewer than 128 workgroups goes on halving down to 960-vector slices.  Measured
-            // per launch, batch 1 / 2 / 4: 960 channels at 64 x 64 (30720 vectors) 8.8 us in
-            // eight against 8.8 in four / 12.3 in eight against 13.4 in four / 21.3 in four
-            // against 23.9 in two; 640 channels at 32 x 32 (5120) 5.12 in four against 5.40 whole /
-            // 5.69 whole against 5.81 in two / 6.10 whole.
-            const size_t whole_limit = units < 64 ? 4096 : 5120;
-            for (;;) {
-                const size_t slice = (vec_per_unit + want - 1) / want;
-                const size_t limit = want == 1 ? whole_limit : units * want < 128 ? 1919 : 5120;
-                if (units * want * 2 > 2 * kChipCus || slice <= limit || slice / 2 < 960 || want >= kGnMaxSplit) break;
-                want *= 2;
-            }
-            // 160 and 192 units (batch 5, 6), as for 2-byte elements: whole up to 10240 vectors, in
-            // four beyond (batch 5 / 6, us: 320 channels at 64 x 64 whole 10.4 / 12.0 against 11.8 /
-            // 12.5 in two, 960 at 32 x 32 8.15 / 9.21 against 9.81 / 10.2; 640 at 64 x 64 in four
-            // 21.2 / 22.5 against 24.5 / 25.7 in two, 960 at 64 x 64 29.9 / 33.5 against 34.4 / 36.6)
-            if (units > 128 && units <= 192 && vec_per_unit > whole_limit) want = vec_per_unit <= 10240 ? 1 : 4;
-        }
-        // 288 ... 384 units (batch 9 - 12): whole units on 1024 lanes would give some CUs two
-        // workgroups and others one; units of 5120 vectors and more are cut into slices of at most
-        // 2560 (5120 from 352 units on), which run as three and more small workgroups per CU (from
-        // 448 units on whole units win again).  Batch 10 / 12, us against
-        // whole: 640 channels at 64 x 64 fp16 22.3 / 23.8 against 26.4 / 26.8, 1920 at 32 x 32 17.7 /
-        // 18.5 against 19.6 / 21.0; 4-byte elements 960 at 32 x 32 15.3 / 17.0 against 17.3 / 20.1,
-        // 320 at 64 x 64 21.4 / 22.4 against 22.5 / 24.0.
-        if (units > kChipCus && units <= 384 && vec_per_unit >= 5120) {
-            if (want < 2) want = 2;
-            const size_t longest = units <= 320 ? 2560 : 5120;  // (batch 12: 23.4 us in two against 23.7 in four)
-            while (vec_per_unit > (size_t)want * longest && want < 8) want *= 2;
-        }
-        // Large batches of very long units (more than 10240 vectors): slices of up to 5120
-        // vectors on 256 lanes overlap better than whole units on 768 - 1024 lanes, the exchange
-        // disappears behind the other workgroups of the CU (batch 32, 15360-vector units: 90 us
-        // in four against 99 us whole)
-        if (units > 384 && vec_per_unit > 10240)
-            while (vec_per_unit > (size_t)want * 2560 && want < 8) want *= 2;
-        // 96 units (batch 3) of more than 96 Ki elements: eight slices are three small workgroups
-        // per CU (960 channels at 64 x 64: 11.2 us against 11.9 in four; 4-byte elements 16.7 against 17.8)
-        if (units == 96 && unit_size > 98304 && want < 8) want = 8;
-        while (units * want < 16 && want < kGnMaxSplit) want *= 2;  // very few units
-        while (split < want && vec_per_unit >= (size_t)2 * split * 256) split *= 2;
-    }
-
-    const size_t vec_per_slice = (vec_per_unit + split - 1) / split;
-    // every slice must own at least one vector (ceil division can starve the last ones)
-    if (vec_per_slice * (split - 1) >= vec_per_unit) return d;
-
-    uint32_t force_threads = 0;
-    if (tune_threads >= kWave && tune_threads <= kGnMaxThreads && tune_threads % kWave == 0 &&
-        (size_t)tune_threads * kMaxK >= vec_per_slice)
-        force_threads = (uint32_t)tune_threads;
-    const bool equal_slices = vec_per_slice * split == vec_per_unit;
-    const GnPlan pl = plan_slice((uint32_t)vec_per_slice, split, force_threads, kMaxK, equal_slices, units * split, elt);
-    if (pl.k == 0 || (pl.k > kGnPrefetchAffineK && cpg > kGnLdsChannels)) return d;
-    d.split = split;
-    d.threads = pl.threads;
-    d.k = (uint32_t)pl.k;
-    d.vec_per_slice = (uint32_t)vec_per_slice;
-    return d;
-}
 
 template <typename T>
 int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma, const float *beta,
@@ -1096,7 +802,7 @@ int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma
     p.writers = d.writers;
     p.writers_shift = (uint32_t)__builtin_ctz(d.writers);
     p.part_vecs = (uint32_t)((((p.vec_per_unit + d.writers - 1) / d.writers + kWave - 1) / kWave) * kWave);
-    p.same_xcd = (shared && units % 8 == 0) ? 1u : 0u;
+    p.xcd_shift = gn_xcd_shift(gn_chip(), shared, units);
 
     GnScratch sc{nullptr, nullptr, nullptr, nullptr, nullptr, 0};
     if (fixed != nullptr) {
@@ -1170,21 +876,17 @@ int gn_tokens_dispatch(const void *xv, void *yv, const float *gamma, const float
                            (cpg * sizeof(T)) % 4 == 0 && (channels * sizeof(T)) % 4 == 0;
     if (!vector_ok) return generic();
     const size_t hw_vec = hw / EPV;
-    // slices cut the positions: the split must divide them, fit the registers and the LDS
-    // (cut earlier than gn_dispatch does: with batch * split = 8 the writers of an output line
-    // share an XCD, which is worth more than the exchange costs from 16 Ki elements on)
+    // slices cut the positions: the split must divide them, fit the registers and the LDS.
+    // Cut earlier than gn_dispatch does: the block layout puts the workgroups that write pieces
+    // of the same output lines on one XCD when batch * split is a multiple of the XCD count, which
+    // is worth more than the exchange costs from 16 Ki elements on.  With half a workgroup per CU
+    // or more, units stay whole or (exactly half) go in two; four slices otherwise, eight when
+    // even that leaves a quarter of the chip idle and a slice keeps 4 Ki elements.
+    const GnChip chip = gn_chip();
     uint32_t want = 1;
     if (unit_size > 16384) {
-        // (more than 128 units: two slices would put two large workgroups on some CUs and one on
-        // others - 640 channels at 32 x 32, batch 5 / 6 / 7: 8.80 / 9.15 / 9.80 us whole against
-        // 9.56 / 10.2 / 10.6 in two)
-        want = units > 128 ? 1 : units >= 128 ? 2 : 4;
-        // (batch 1, 320 channels at 64 x 64: 6.59 us in eight against 7.16 in four, 4-byte elements
-        // 7.45 against 8.45)
-        if (units * 4 < 192 && unit_size >= 32768) want = 8;
-        // (288 and 320 units of 32 Ki elements and more: batch 10, 320 channels at 64 x 64 25.2 us
-        // in four against 29.4 whole; from 384 units on whole units win)
-        if (units > 256 && units <= 320 && unit_size >= 32768) want = 4;
+        want = units * 2 > chip.cus ? 1 : units * 2 == chip.cus ? 2 : 4;
+        if (units * 16 < 3 * (size_t)chip.cus && unit_size >= 32768) want = 8;
     }
     const int tune_split = g_tuning.gn_split.load(std::memory_order_relaxed);
     const int tune_spin = g_tuning.gn_spin_limit.load(std::memory_order_relaxed);
@@ -1208,7 +910,7 @@ int gn_tokens_dispatch(const void *xv, void *yv, const float *gamma, const float
     const size_t bytes = units * unit_size * sizeof(T);
     const bool apart = xb + bytes <= yb || yb + bytes <= xb;
     if (apart && tune_split <= 1 && tune_writers != 1 && vec_per_unit <= (size_t)kGnMaxThreads * kGnSharedMaxK) {
-        uint32_t w = tune_writers > 1 ? (uint32_t)tune_writers : gn_auto_writers(sizeof(T), units, vec_per_unit);
+        uint32_t w = tune_writers > 1 ? (uint32_t)tune_writers : gn_auto_writers(chip, sizeof(T), units, vec_per_unit);
         // Here the limit is lower than for the channel-major store: the slices of a cut unit
         // also keep the writers of an output line on one XCD, which the writers of a unit give
         // up.  Measured, batch 2 fp16, several writers against slices: 1280 channels at 16 x 16
@@ -1223,7 +925,7 @@ int gn_tokens_dispatch(const void *xv, void *yv, const float *gamma, const float
         }
         writers = (w < 1 || units * w > 0x7FFFFFFFull) ? 1 : w;  // (the grid is units * writers blocks)
         if (writers > 1 &&
-            plan_slice((uint32_t)vec_per_unit, 1, 0, kGnSharedMaxK, true, units * writers, sizeof(T)).k == 0)
+            gn_threads_for(chip, sizeof(T), (uint32_t)vec_per_unit, 1, units * writers, kGnSharedMaxK, true, true).k == 0)
             writers = 1;  // (the whole unit does not fit one workgroup's registers: slices as below)
     }
     const bool shared = writers > 1;
@@ -1240,7 +942,7 @@ int gn_tokens_dispatch(const void *xv, void *yv, const float *gamma, const float
     q.base.writers = writers;
     q.base.writers_shift = (uint32_t)__builtin_ctz(writers);
     q.base.part_vecs = (uint32_t)nvec;
-    q.base.same_xcd = (shared && units % 8 == 0) ? 1u : 0u;
+    q.base.xcd_shift = gn_xcd_shift(chip, shared, units);
     q.base.groups = (uint32_t)groups;
     q.base.ch_per_group = (uint32_t)cpg;
     q.base.hw_vec = make_fast_div((uint32_t)hw_vec);
@@ -1256,8 +958,9 @@ int gn_tokens_dispatch(const void *xv, void *yv, const float *gamma, const float
     q.part_len = make_fast_div((uint32_t)nvec);
     const size_t lds_bytes = cpg * q.pitch * sizeof(T);
     // a workgroup holds its slice, or with several writers the whole unit
-    const GnPlan pl = shared ? plan_slice((uint32_t)vec_per_unit, 1, 0, kGnSharedMaxK, true, units * writers, sizeof(T))
-                             : plan_slice((uint32_t)nvec, split, 0, kMaxK, false);
+    const GnThreads pl = shared ? gn_threads_for(chip, sizeof(T), (uint32_t)vec_per_unit, 1, units * writers, kGnSharedMaxK,
+                                                 true, true)
+                                : gn_threads_for(chip, sizeof(T), (uint32_t)nvec, split, units * split, kMaxK, false, false);
     if (pl.k == 0) return generic();
     GnScratch sc{nullptr, nullptr, nullptr, nullptr, nullptr, 0};
     if (!shared && split > 1) {

@@ -47,6 +47,14 @@ inline int launch_status() {
 constexpr uint32_t kGnMaxSplit = 64;    // workgroups per unit (one wavefront reads all slots)
 constexpr uint32_t kGnMaxUnits = 8192;  // units that own scratch slots; larger launches never split
 
+// ---- what the GroupNorm register kernels are built for (kernels: groupnorm.hip, plan: gn_plan.hip) ----
+constexpr int kGnMaxThreads = 1024;
+constexpr int kGnMaxK = 20;             // vectors per lane; the largest only for slices it fits exactly
+constexpr int kGnMaxRaggedK = 16;       // the largest with code for a ragged slice
+constexpr int kGnSharedMaxK = 10;       // kernels with several writers per unit exist up to this many vectors per lane
+constexpr int kGnPrefetchAffineK = 6;   // vectors per lane up to which gamma / beta are kept in registers
+constexpr uint32_t kGnLdsChannels = 1024;  // channels per group the LDS copy of gamma / beta has room for
+
 struct GnScratch {
     unsigned long long *slot_mean;  // [kGnMaxUnits][kGnMaxSplit]  (tag << 32) | float bits
     unsigned long long *slot_m2;    // [kGnMaxUnits][kGnMaxSplit]
@@ -73,10 +81,13 @@ struct Tuning {
     std::atomic<int> act_vectors{0};
     std::atomic<int> softmax_rows{0};
     std::atomic<int> gn_spin_limit{0};
+    std::atomic<int> device_cus{0};
+    std::atomic<int> device_xcds{0};
+    std::atomic<int> gn_plan_rule_only{0};
 };
 extern Tuning g_tuning;
 
-// The launch msd_groupnorm makes for a shape (see gn_decide in groupnorm.hip): split == 0 is the
+// The launch msd_groupnorm makes for a shape (see gn_decide in gn_plan.hip): split == 0 is the
 // general kernel, otherwise split workgroups of `threads` lanes per (sample, group), k 16-byte
 // vectors per lane, vec_per_slice vectors per workgroup.
 struct GnDecision {
@@ -88,6 +99,22 @@ struct GnDecision {
 };
 GnDecision gn_decide(size_t elt, size_t batch, size_t channels, size_t hw, size_t groups, bool aligned,
                      size_t max_units, bool may_share);
+
+// Compute units and XCDs of the current device (gn_plan.hip; the knobs can replace them).
+struct GnChip {
+    uint32_t cus;
+    uint32_t xcds;
+};
+GnChip gn_chip();
+// Lanes and vectors per lane (k == 0: none fits) for a workgroup that holds `vecs` vectors.
+struct GnThreads {
+    uint32_t threads;
+    int k;
+};
+int gn_k_for(uint32_t vecs, uint32_t threads, uint32_t max_k, bool equal_slices);
+GnThreads gn_threads_for(const GnChip &chip, size_t elt, uint32_t vecs, uint32_t split, size_t blocks, uint32_t max_k,
+                         bool equal_slices, bool shared);
+uint32_t gn_auto_writers(const GnChip &chip, size_t elt, size_t units, size_t vec_per_unit);
 
 // ---- per-dtype dispatchers (T = float or __half), defined in the kernel files ----
 // fixed: scratch to use instead of the stream's own (units beyond its capacity are refused)

@@ -73,9 +73,10 @@ def test_argument_validation_needs_no_gpu(msd):
     assert lib.msd_set_tuning(1, 100) == 1    # threads must be a multiple of 64
     assert lib.msd_set_tuning(2, 12) == 1 and lib.msd_set_tuning(4, 3) == 1 and lib.msd_set_tuning(99, 1) == 1
     assert lib.msd_set_tuning(6, 48) == 1     # softmax rows per workgroup: 16, 32 or 64
-    assert lib.msd_set_tuning(9, 0) == 1      # no such knob
+    assert lib.msd_set_tuning(12, 0) == 1     # no such knob
     assert lib.msd_set_tuning(8, 3) == 1 and lib.msd_set_tuning(8, 32) == 1   # writers: a power of two up to 16
-    for knob in range(9):
+    assert lib.msd_set_tuning(9, 5000) == 1 and lib.msd_set_tuning(10, 65) == 1 and lib.msd_set_tuning(11, 2) == 1
+    for knob in range(12):
         assert lib.msd_set_tuning(knob, 0) == 0
     # GEGLU rows of input and output have different strides: any overlap is refused
     # (addresses are never dereferenced: the check comes before the launch)

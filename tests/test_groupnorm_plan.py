@@ -47,20 +47,66 @@ def _check(batch, channels, hw, groups, code, noalloc=False, in_place=False):
     return split, threads, k, writers
 
 
-def test_plans_at_the_batches_in_between():
-    """Between one and two workgroups per CU the plan keeps units whole or cuts them into many small
-    slices, never into one to two 1024-lane workgroups per CU (the measured rules of gn_decide)."""
-    f16, f32 = msd.DTYPE_F16, msd.DTYPE_F32
-    in_place = {
-        (3, 320, 4096, f16): (2, 1024, 3, 1), (3, 960, 4096, f16): (8, 512, 4, 1),
-        (5, 320, 4096, f16): (1, 1024, 5, 1), (6, 640, 4096, f16): (4, 512, 5, 1), (7, 960, 4096, f16): (1, 1024, 16, 1),
-        (5, 960, 1024, f32): (1, 768, 10, 1), (6, 1920, 1024, f32): (4, 512, 8, 1), (7, 640, 1024, f32): (1, 512, 10, 1),
-        (10, 640, 4096, f16): (4, 256, 10, 1), (12, 640, 4096, f16): (2, 512, 10, 1), (10, 320, 4096, f32): (4, 256, 10, 1),
-        (14, 320, 4096, f16): (1, 1024, 5, 1), (16, 640, 1024, f16): (1, 512, 5, 1), (24, 640, 4096, f32): (8, 512, 5, 1),
-        (24, 640, 1024, f16): (1, 256, 10, 1),
-    }
-    for (batch, channels, hw, code), want in in_place.items():
-        assert _check(batch, channels, hw, 32, code, in_place=True) == want, (batch, channels, hw, code)
+UNET_SHAPES = [(1280, 64), (640, 256), (2560, 64), (320, 1024), (1280, 256), (1920, 256), (640, 1024), (2560, 256),
+               (960, 1024), (320, 4096), (1280, 1024), (1920, 1024), (640, 4096), (960, 4096)]   # (channels, hw)
+
+
+def _knobs(msd, **values):
+    lib = msd.load_library()
+    for name, value in values.items():
+        assert lib.msd_set_tuning(getattr(msd, "TUNE_" + name), value) == 0
+
+
+def test_the_rule_alone_plans_every_batch_and_keeps_a_cu_per_workgroup_when_it_cuts_units():
+    """With the table of measured plans switched off, every UNet shape at every batch from 1 to 40
+    gets a launch that fits; and while there are fewer units than CUs the rule cuts units only as
+    long as every slice still has a CU to itself (two slices per CU for 4-byte elements), unless
+    the registers of one workgroup cannot hold the unit."""
+    _knobs(msd, GN_PLAN_RULE_ONLY=1)
+    try:
+        for batch in range(1, 41):
+            for channels, hw in UNET_SHAPES:
+                for code, elt in ((msd.DTYPE_F16, 2), (msd.DTYPE_F32, 4)):
+                    for in_place in (True, False):
+                        split, threads, k, writers = _check(batch, channels, hw, 32, code, in_place=in_place)
+                        units, vecs = batch * 32, channels // 32 * hw * elt // 16
+                        if split > 1 and units < 256 and vecs <= 16 * 1024:
+                            assert units * split <= (256 if elt == 2 else 512), (batch, channels, hw, elt, split)
+                        if writers > 1:
+                            assert units * writers <= 256 and units % 8 == 0
+    finally:
+        _knobs(msd, GN_PLAN_RULE_ONLY=0)
+
+
+def test_plans_follow_the_chip_that_is_reported():
+    """CU and XCD counts come from the device (here: injected through the knobs).  The table of
+    measured plans belongs to 256 CUs in 8 XCDs and is not consulted elsewhere; writers per unit
+    follow the CU count, need the units in whole rows of a power-of-two XCD count, and a chip of
+    one XCD needs no such rows."""
+    f16 = msd.DTYPE_F16
+    try:
+        # the chip the table was measured on: the measured plan of 320 channels at 64 x 64, batch 2, in place
+        assert msd.groupnorm_plan(2, 320, 4096, 32, f16, in_place=True) == (4, 640, 2, 1)
+        _knobs(msd, DEVICE_CUS=64, DEVICE_XCDS=2)     # a quarter of the chip
+        assert msd.groupnorm_plan(2, 320, 4096, 32, f16, in_place=True) == (1, 1024, 5, 1)   # 64 units on 64 CUs: whole
+        assert msd.groupnorm_plan(1, 640, 1024, 32, f16)[3] == 2     # 32 units: two writers fill 64 CUs
+        assert msd.groupnorm_plan(2, 640, 1024, 32, f16)[3] == 1     # 64 units: every CU has a unit already
+        _knobs(msd, DEVICE_CUS=228, DEVICE_XCDS=6)    # not a power of two: no block-id stride keeps writers on one XCD
+        assert msd.groupnorm_plan(1, 640, 1024, 32, f16)[3] == 1
+        _knobs(msd, DEVICE_CUS=304, DEVICE_XCDS=8)    # more CUs than the table's chip: the rule, same shape of plan
+        assert msd.groupnorm_plan(1, 640, 1024, 32, f16)[3] == 8 and msd.groupnorm_plan(4, 640, 1024, 32, f16)[3] == 2
+        _knobs(msd, DEVICE_CUS=32, DEVICE_XCDS=1)     # one XCD (a partitioned device): no rows of units needed
+        assert msd.groupnorm_plan(1, 24, 4096, 3, f16)[3] == 8       # 3 units, one L2 for everybody
+        _knobs(msd, DEVICE_CUS=256, DEVICE_XCDS=8)
+        assert msd.groupnorm_plan(3, 24, 4096, 3, f16)[3] == 1       # 9 units on 8 XCDs: the writers would sit apart
+        for cus, xcds in ((16, 1), (64, 2), (120, 4), (228, 6), (1024, 16)):   # whatever the chip, a launch that fits
+            _knobs(msd, DEVICE_CUS=cus, DEVICE_XCDS=xcds)
+            for batch in (1, 2, 5, 32):
+                for channels, hw in UNET_SHAPES:
+                    _check(batch, channels, hw, 32, f16)
+                    _check(batch, channels, hw, 32, msd.DTYPE_F32, in_place=True)
+    finally:
+        _knobs(msd, DEVICE_CUS=0, DEVICE_XCDS=0)
 
 
 def test_plans_of_the_unet_shapes_at_batch_2_and_32():
@@ -83,7 +129,7 @@ def test_plans_of_the_unet_shapes_at_batch_2_and_32():
         (2, 320, 4096, f16): (1, 1024, 5, 4), (2, 640, 1024, f16): (1, 640, 4, 4), (2, 1280, 256, f16): (1, 512, 3, 4),
         (2, 1280, 64, f16): (1, 384, 1, 4), (2, 960, 1024, f16): (1, 1024, 4, 4), (2, 1920, 256, f16): (1, 512, 4, 4),
         (2, 1920, 1024, f16): (4, 960, 2, 1), (2, 640, 4096, f16): (4, 1024, 3, 1),
-        (1, 320, 4096, f16): (1, 1024, 5, 8), (1, 1280, 64, f16): (1, 384, 1, 4), (4, 640, 1024, f16): (1, 640, 4, 2),
+        (1, 320, 4096, f16): (1, 1024, 5, 8), (1, 1280, 64, f16): (1, 384, 1, 4), (4, 640, 1024, f16): (1, 1024, 3, 2),
         (1, 320, 4096, f32): (4, 640, 4, 1), (1, 640, 1024, f32): (1, 1024, 5, 8), (2, 320, 4096, f32): (1, 1024, 10, 4),
         (2, 960, 1024, f32): (1, 1024, 8, 4), (2, 960, 4096, f32): (8, 960, 4, 1), (2, 1280, 256, f32): (1, 640, 4, 4),
         (8, 320, 4096, f16): (1, 1024, 5, 1), (32, 320, 4096, f16): (1, 256, 20, 1),
