@@ -34,6 +34,13 @@ inline int round_up_k(uint32_t k) {
 // K = 10 / 12 / 16 / 20 need 74 / 85 / 120 / 121 - the compiler's resource report).
 inline uint32_t waves_per_simd(int k) { return k <= 8 ? 8u : k == 10 ? 6u : k == 12 ? 5u : 4u; }
 
+// All `blocks` workgroups of `threads` lanes are on the chip at once: a workgroup puts a quarter of
+// its wavefronts (rounded up) on each of a CU's four SIMDs.
+inline bool launch_is_resident(const Chip &chip, size_t blocks, uint32_t threads, int k) {
+    const uint32_t per_simd = (threads / kWave + 3) / 4;
+    return blocks <= (size_t)chip.cus * (waves_per_simd(k) / per_simd);
+}
+
 // Relative cost of holding a slice as K vectors per lane when a workgroup has a CU to itself
 // (measured on whole units of 1280 ... 15360 vectors, one workgroup per CU, against the best
 // size for the same unit): 1, 2, 3, 5 cost nothing, 10 and 20 little, 4 / 6 / 8 / 12 / 16 lose
@@ -96,10 +103,10 @@ int gn_k_for(uint32_t vecs, uint32_t threads, uint32_t max_k, bool equal_slices)
 // workgroups to the XCDs in turn; each XCD has an L2 of its own).  Asked once per device; the
 // knobs MSD_TUNE_DEVICE_CUS / _XCDS replace the answer (tests plan for other chips with them);
 // without a device (planning on a host that has none) the MI355X's 256 CUs in 8 XCDs.
-GnChip gn_chip() {
+Chip chip_info() {
     constexpr int kMaxDevices = 64;
     static std::atomic<uint32_t> cached[kMaxDevices];  // (cus << 8) | xcds, 0 = not asked yet
-    GnChip chip{256, 8};
+    Chip chip{256, 8};
     int device = 0;
     if (hipGetDevice(&device) == hipSuccess && device >= 0 && device < kMaxDevices) {
         uint32_t packed = cached[device].load(std::memory_order_relaxed);
@@ -111,7 +118,7 @@ GnChip gn_chip() {
                 cached[device].store(packed, std::memory_order_relaxed);
             }
         }
-        if (packed != 0) chip = GnChip{packed >> 8, packed & 255u};
+        if (packed != 0) chip = Chip{packed >> 8, packed & 255u};
     } else {
         (void)hipGetLastError();  // no device: not an error of the caller's
     }
@@ -129,7 +136,7 @@ GnChip gn_chip() {
 // a w-th while nothing is exchanged.  w = as many as give the chip one workgroup per CU, 8 at
 // most.  Past 5120 vectors of 2-byte elements (10240 of 4-byte ones, 5120 with eight writers)
 // the repeated loads cost more than the shorter epilogue gains.
-uint32_t gn_auto_writers(const GnChip &chip, size_t elt, size_t units, size_t vec_per_unit) {
+uint32_t gn_auto_writers(const Chip &chip, size_t elt, size_t units, size_t vec_per_unit) {
     // The writers of a unit must run on one XCD (block ids a multiple of the XCD count apart),
     // which needs a power-of-two XCD count and the units in whole rows of that many; on
     // different XCDs every copy of the loads comes from memory and the launch is slower than
@@ -144,29 +151,37 @@ uint32_t gn_auto_writers(const GnChip &chip, size_t elt, size_t units, size_t ve
 // Lanes and K for a workgroup that holds `vecs` vectors in a launch of `blocks` workgroups.
 // `split`: slices per unit of the launch; `shared`: every workgroup holds a whole unit that
 // several of them finish.
-GnThreads gn_threads_for(const GnChip &chip, size_t elt, uint32_t vecs, uint32_t split, size_t blocks, uint32_t max_k,
+GnThreads gn_threads_for(const Chip &chip, size_t elt, uint32_t vecs, uint32_t split, size_t blocks, uint32_t max_k,
                          bool equal_slices, bool shared) {
     GnThreads pl{0, 0};
     auto k_of = [&](uint32_t t) { return gn_k_for(vecs, t, max_k, equal_slices); };
     if (blocks > chip.cus) {
         // Throughput: the CUs hold several workgroups each, in different phases (load, statistics,
-        // store).  Slices of cut units take the smallest workgroup that holds them in at most
-        // five vectors per lane (eight wavefronts per SIMD).  Otherwise the smallest of 256 ...
-        // 1024 lanes that holds the unit - fewer, longer wavefronts, a barrier that joins four of
-        // them instead of sixteen, and the whole launch resident at once (K = 20 on 256 lanes:
-        // four wavefronts per workgroup, four per SIMD) - as long as short units still give every
-        // CU ten wavefronts to hide latency with.
-        if (split > 1)
+        // store).  The smallest of 256 ... 1024 lanes that holds the unit (512 ... for slices of cut
+        // units) - fewer, longer wavefronts, a barrier that joins four of them instead of sixteen,
+        // and the whole launch resident at once (K = 20 on 256 lanes: four wavefronts per
+        // workgroup, four per SIMD) - as long as short units still give every CU ten wavefronts to
+        // hide latency with.  From eight workgroups per CU on, slices of cut units take the
+        // smallest workgroup that holds them in at most five vectors per lane instead (eight
+        // wavefronts per SIMD).
+        if (split > 1 && blocks >= 8 * (size_t)chip.cus)
             for (uint32_t t = 256; t <= kGnMaxThreads && pl.threads == 0; t += kWave) {
                 const int k = k_of(t);
                 if (k != 0 && k <= 5) pl.threads = t;
             }
+        uint32_t smallest = 0;
         for (uint32_t t = 256; t <= kGnMaxThreads && pl.threads == 0; t += 256) {
             if (k_of(t) == 0 || (split > 1 && t == 256)) continue;
+            if (smallest == 0) smallest = t;
             if (vecs <= 4096 && blocks * (t / kWave) < 10 * (size_t)chip.cus && t < kGnMaxThreads) continue;
             pl.threads = t;
         }
         if (pl.threads == 0) pl.threads = kGnMaxThreads;
+        // (more wavefronts per CU are not worth a launch that no longer fits the chip at once)
+        if (smallest != 0 && smallest != pl.threads && k_of(pl.threads) != 0 &&
+            !launch_is_resident(chip, blocks, pl.threads, k_of(pl.threads)) &&
+            launch_is_resident(chip, blocks, smallest, k_of(smallest)))
+            pl.threads = smallest;
     } else if (shared && vecs <= 2560) {
         // every writer reduces the whole unit and a part of its wavefronts does the epilogue:
         // fewer lanes with more vectors each than a lone workgroup would take
@@ -197,7 +212,7 @@ GnThreads gn_threads_for(const GnChip &chip, size_t elt, uint32_t vecs, uint32_t
 namespace {
 
 // Slices per unit the rule wants for whole units of `vec_per_unit` vectors (1: whole).
-uint32_t rule_split(const GnChip &chip, size_t elt, size_t units, size_t vec_per_unit) {
+uint32_t rule_split(const Chip &chip, size_t elt, size_t units, size_t vec_per_unit) {
     const size_t epv = 16 / elt;
     const size_t slice = kSliceElements / epv;  // vectors
     uint32_t want = 1;
@@ -222,6 +237,17 @@ uint32_t rule_split(const GnChip &chip, size_t elt, size_t units, size_t vec_per
         // workgroups of the CU.
         while (vec_per_unit > (size_t)want * 2560 && want < 8) want *= 2;
     }
+    // Between one and two workgroups per CU a launch runs as two rounds with the second mostly
+    // empty.  Slices of units shorter than three times the size above are merged back (a CU each,
+    // or nearly); longer units, and whole units from twice that size on, are cut once more (two
+    // and more workgroups on every CU).
+    const size_t blocks = units * want;
+    if (blocks > chip.cus && blocks < 2 * (size_t)chip.cus) {
+        if (want > 1 && vec_per_unit < 3 * slice)
+            want /= 2;
+        else if (vec_per_unit >= 2 * slice && want < 8)
+            want *= 2;
+    }
     while (units * want < 16 && want < kGnMaxSplit) want *= 2;  // very few units
     return want;
 }
@@ -244,7 +270,7 @@ GnDecision gn_decide(size_t elt, size_t batch, size_t channels, size_t hw, size_
     // (the register kernel addresses a unit with 32-bit byte offsets)
     if (!aligned || hw % epv != 0 || unit_size * elt >= (1ull << 32)) return d;
     const size_t vec_per_unit = unit_size / epv;
-    const GnChip chip = gn_chip();
+    const Chip chip = chip_info();
 
     const int tune_split = g_tuning.gn_split.load(std::memory_order_relaxed);
     const int tune_threads = g_tuning.gn_threads.load(std::memory_order_relaxed);

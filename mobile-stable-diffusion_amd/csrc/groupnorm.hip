@@ -723,7 +723,7 @@ __global__ __launch_bounds__(kGenericThreads) void gn_tokens_generic_kernel(
 // log2 of the distance between the block ids of a unit's writers: the XCD count when the
 // workgroups of a launch are dealt to a power-of-two number of XCDs in turn and the units come
 // in whole rows of that many (the writers then share an XCD), else 0 (adjacent ids).
-inline uint32_t gn_xcd_shift(const GnChip &chip, bool shared, size_t units) {
+inline uint32_t gn_xcd_shift(const Chip &chip, bool shared, size_t units) {
     if (!shared || chip.xcds <= 1 || (chip.xcds & (chip.xcds - 1)) != 0 || units % chip.xcds != 0) return 0;
     return (uint32_t)__builtin_ctz(chip.xcds);
 }
@@ -802,7 +802,7 @@ int gn_dispatch(const void *xv, const void *chunkv, void *yv, const float *gamma
     p.writers = d.writers;
     p.writers_shift = (uint32_t)__builtin_ctz(d.writers);
     p.part_vecs = (uint32_t)((((p.vec_per_unit + d.writers - 1) / d.writers + kWave - 1) / kWave) * kWave);
-    p.xcd_shift = gn_xcd_shift(gn_chip(), shared, units);
+    p.xcd_shift = gn_xcd_shift(chip_info(), shared, units);
 
     GnScratch sc{nullptr, nullptr, nullptr, nullptr, nullptr, 0};
     if (fixed != nullptr) {
@@ -882,7 +882,7 @@ int gn_tokens_dispatch(const void *xv, void *yv, const float *gamma, const float
     // is worth more than the exchange costs from 16 Ki elements on.  With half a workgroup per CU
     // or more, units stay whole or (exactly half) go in two; four slices otherwise, eight when
     // even that leaves a quarter of the chip idle and a slice keeps 4 Ki elements.
-    const GnChip chip = gn_chip();
+    const Chip chip = chip_info();
     uint32_t want = 1;
     if (unit_size > 16384) {
         want = units * 2 > chip.cus ? 1 : units * 2 == chip.cus ? 2 : 4;

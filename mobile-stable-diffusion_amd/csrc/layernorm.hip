@@ -257,12 +257,12 @@ __global__ __launch_bounds__(kLnThreads) void ln_generic_kernel(
 template <typename T, int NW, int VPL, int TL>
 void ln_launch(const T *x, const T *res, T *sum, T *y, const float *gamma, const float *beta,
                uint32_t rows, float eps, float inv_dim, hipStream_t stream) {
-    // Up to one wavefront per SIMD of the chip (1024) the launch is bound by its own latency chain:
+    // Up to one wavefront per SIMD of the chip (four SIMDs per CU) the launch is bound by its own latency chain:
     // one wavefront per workgroup (1 - 5 % faster than four), gamma / beta requested together with
     // the row.  From two wavefronts per SIMD on throughput counts: gamma / beta through LDS (fewer
     // load instructions and registers per wavefront), four wavefronts per workgroup, two for
-    // launches of 4096 up to 10240 wavefronts (3 - 19 % faster there, 1 - 7 % slower at 3072 and
-    // from 10240 on).  Measured, us per launch, with the row / LDS x 64, 128, 256 lanes:
+    // launches of four up to ten wavefronts per SIMD (3 - 19 % faster there, 1 - 7 % slower at three
+    // and from ten on).  Measured, us per launch, with the row / LDS x 64, 128, 256 lanes:
     //   fp16 8192 x 320 (1024 wavefronts)   3.54 3.71 3.59 / 3.57 3.88 3.57
     //   fp16 16384 x 320 (2048)             5.12 5.19 5.22 / 4.94 4.78 4.94
     //   fp32 8192 x 320 (2048)              5.28 5.29 5.17 / 4.90 4.71 4.99
@@ -271,11 +271,12 @@ void ln_launch(const T *x, const T *res, T *sum, T *y, const float *gamma, const
     //   fp16 8192 x 1280 (4096)             10.4 10.6 10.4 / 8.19 7.95 7.95
     //   fp16 32768 x 1024 (32768)           24.5 24.5 24.5 / 31.7 25.0 24.1
     const uint32_t wavefronts = (rows + (kWave / TL) - 1) / (kWave / TL);
-    const bool early = wavefronts < 2048;
+    const uint32_t simds = 4 * chip_info().cus;  // (the figures above: 1024 SIMDs)
+    const bool early = wavefronts < 2 * simds;
     const int tune_threads = g_tuning.ln_threads.load(std::memory_order_relaxed);
     const uint32_t threads = tune_threads ? (uint32_t)tune_threads
-                             : early      ? (wavefronts <= 1024 ? (uint32_t)kLnThreads : 256u)
-                                          : (wavefronts >= 4096 && wavefronts < 10240 ? 128u : 256u);
+                             : early      ? (wavefronts <= simds ? (uint32_t)kLnThreads : 256u)
+                                          : (wavefronts >= 4 * simds && wavefronts < 10 * simds ? 128u : 256u);
     const uint32_t rows_per_block = (kWave / TL) * (threads / kWave);
     const uint32_t blocks = (rows + rows_per_block - 1) / rows_per_block;
     if (early)

@@ -101,20 +101,20 @@ GnDecision gn_decide(size_t elt, size_t batch, size_t channels, size_t hw, size_
                      size_t max_units, bool may_share);
 
 // Compute units and XCDs of the current device (gn_plan.hip; the knobs can replace them).
-struct GnChip {
+struct Chip {
     uint32_t cus;
     uint32_t xcds;
 };
-GnChip gn_chip();
+Chip chip_info();
 // Lanes and vectors per lane (k == 0: none fits) for a workgroup that holds `vecs` vectors.
 struct GnThreads {
     uint32_t threads;
     int k;
 };
 int gn_k_for(uint32_t vecs, uint32_t threads, uint32_t max_k, bool equal_slices);
-GnThreads gn_threads_for(const GnChip &chip, size_t elt, uint32_t vecs, uint32_t split, size_t blocks, uint32_t max_k,
+GnThreads gn_threads_for(const Chip &chip, size_t elt, uint32_t vecs, uint32_t split, size_t blocks, uint32_t max_k,
                          bool equal_slices, bool shared);
-uint32_t gn_auto_writers(const GnChip &chip, size_t elt, size_t units, size_t vec_per_unit);
+uint32_t gn_auto_writers(const Chip &chip, size_t elt, size_t units, size_t vec_per_unit);
 
 // ---- per-dtype dispatchers (T = float or __half), defined in the kernel files ----
 // fixed: scratch to use instead of the stream's own (units beyond its capacity are refused)

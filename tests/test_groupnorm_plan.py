@@ -57,11 +57,11 @@ def _knobs(msd, **values):
         assert lib.msd_set_tuning(getattr(msd, "TUNE_" + name), value) == 0
 
 
-def test_the_rule_alone_plans_every_batch_and_keeps_a_cu_per_workgroup_when_it_cuts_units():
+def test_the_rule_alone_plans_every_batch_and_never_leaves_cut_units_between_one_and_two_workgroups_per_cu():
     """With the table of measured plans switched off, every UNet shape at every batch from 1 to 40
-    gets a launch that fits; and while there are fewer units than CUs the rule cuts units only as
-    long as every slice still has a CU to itself (two slices per CU for 4-byte elements), unless
-    the registers of one workgroup cannot hold the unit."""
+    gets a launch that fits; and when the rule cuts units (it is not the registers of one workgroup
+    that force it) the launch has at most one workgroup per CU or at least two, never one and a
+    bit: such a launch runs as two rounds with the second mostly empty."""
     _knobs(msd, GN_PLAN_RULE_ONLY=1)
     try:
         for batch in range(1, 41):
@@ -70,8 +70,8 @@ def test_the_rule_alone_plans_every_batch_and_keeps_a_cu_per_workgroup_when_it_c
                     for in_place in (True, False):
                         split, threads, k, writers = _check(batch, channels, hw, 32, code, in_place=in_place)
                         units, vecs = batch * 32, channels // 32 * hw * elt // 16
-                        if split > 1 and units < 256 and vecs <= 16 * 1024:
-                            assert units * split <= (256 if elt == 2 else 512), (batch, channels, hw, elt, split)
+                        if split > 1 and vecs <= 16 * 1024:
+                            assert not 256 < units * split < 512, (batch, channels, hw, elt, split)
                         if writers > 1:
                             assert units * writers <= 256 and units % 8 == 0
     finally:
@@ -131,7 +131,8 @@ def test_plans_of_the_unet_shapes_at_batch_2_and_32():
         (2, 1920, 1024, f16): (4, 960, 2, 1), (2, 640, 4096, f16): (4, 1024, 3, 1),
         (1, 320, 4096, f16): (1, 1024, 5, 8), (1, 1280, 64, f16): (1, 384, 1, 4), (4, 640, 1024, f16): (1, 1024, 3, 2),
         (1, 320, 4096, f32): (4, 640, 4, 1), (1, 640, 1024, f32): (1, 1024, 5, 8), (2, 320, 4096, f32): (1, 1024, 10, 4),
-        (2, 960, 1024, f32): (1, 1024, 8, 4), (2, 960, 4096, f32): (8, 960, 4, 1), (2, 1280, 256, f32): (1, 640, 4, 4),
+        # (960 channels at 32 x 32, fp32: 768 x 10 measured 5.84 us against 6.04 us for the 1024 x 8 it had before)
+        (2, 960, 1024, f32): (1, 768, 10, 4), (2, 960, 4096, f32): (8, 960, 4, 1), (2, 1280, 256, f32): (1, 640, 4, 4),
         (8, 320, 4096, f16): (1, 1024, 5, 1), (32, 320, 4096, f16): (1, 256, 20, 1),
     }
     for (batch, channels, hw, code), want in apart.items():
