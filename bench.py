@@ -10,7 +10,7 @@ each layer on its own HBM-resident buffers, launched back to back on one stream.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode graph|eager] [--no-cpu] [--no-shapes]
                     [--tables shapes,gn_split,fusions,neighbours,large_batch,gn_plan_sweep]
     python bench.py --sweep-summary OUT.json[,...]               (no GPU: markdown of gn_plan_sweep rows)
-    python bench.py --trace-summary TRACE.csv --bench-json OUT   (no GPU: shapes rows next to a kernel trace)
+    python bench.py --trace-summary TRACE.csv --bench-json OUT [--plain-json OUT2]   (no GPU: shapes rows next to a kernel trace)
 
 Prints ONE JSON line (see the keys below).  The CPU oracle is used only for the
 `cpu_baseline` leg.
@@ -504,10 +504,14 @@ def gn_split_table(torch, msd, dev, stream):
                 writers_us = round(_rotating_launch_us(torch, msd, stream, case["launch"], case["xs"], case["ys"],
                                                        budget=1000), 3)
                 assert lib.msd_set_tuning(msd.TUNE_GN_WRITERS, 1) == 0
+                code = msd.DTYPE_F16 if case["elt"] == 2 else msd.DTYPE_F32
                 for split in (0, 1, 2, 4, 8):
                     for threads in ((0,) if split == 0 else (512, 1024)):
                         assert lib.msd_set_tuning(msd.TUNE_GN_SPLIT, split) == 0
                         assert lib.msd_set_tuning(msd.TUNE_GN_THREADS, threads) == 0
+                        plan = msd.groupnorm_plan(BATCH, c, side * side, 32, code, in_place=True)
+                        if split and (plan[0] != split or plan[1] != threads):
+                            continue  # (the launch cannot follow this setting: slices too short, registers)
                         key = "auto" if split == 0 else "s%d_t%d" % (split, threads)
                         times[key] = round(_rotating_launch_us(torch, msd, stream, case["launch"], case["xs"],
                                                                case["ys"], budget=1000), 3)
@@ -657,7 +661,7 @@ def sweep_summary(paths):
     return "\n".join(out)
 
 
-def trace_summary(trace_csv, bench_json):
+def trace_summary(trace_csv, bench_json, plain_json=None):
     """Markdown table: the rows of the `shapes` table of a profiled bench.py run next to the
     device durations rocprofv3 --kernel-trace recorded for them.  The run's trace is cut at the
     marker launches (TraceMarkers) whose labels the bench line carries in `trace_markers`; inside
@@ -695,11 +699,18 @@ def trace_summary(trace_csv, bench_json):
         return name
 
     rows = bench["shapes"]
-    out = ["| config | kernel | shape | dtype | measurement | bytes | bench.py us (graph chain) | profiled kernel | grid x workgroup | dispatches | "
-           "median device us | GB/s at that | frac of 8 TB/s |", "|---|---|---|---|---|---:|---:|---|---|---:|---:|---:|---:|"]
+    plain = None  # the same table from a run without the profiler, when given
+    if plain_json:
+        with open(plain_json) as f:
+            for line in f:
+                if line.startswith("{"):
+                    plain = json.loads(line)["shapes"]
+    out = ["| config | kernel | shape | dtype | measurement | bytes | bench.py us per launch, graph chain: unprofiled run | this profiled run | "
+           "profiled kernel | workgroups x lanes | dispatches | median device us | GB/s at that | frac of 8 TB/s |",
+           "|---|---|---|---|---|---:|---:|---:|---|---|---:|---:|---:|---:|"]
     for i, lab in enumerate(labels):
         found = cuts.get(i, [])
-        if not found or lab["what"] == "memcpy_us":
+        if not found:  # (the runtime's memcpy shows up here only when it runs as a kernel)
             continue
         groups = {}
         for name, grid, wg, dur in found:
@@ -710,8 +721,11 @@ def trace_summary(trace_csv, bench_json):
         row = rows[lab["row"]]
         shape = " ".join("%s=%s" % kv for kv in row["shape"].items())
         gbs = lab["bytes"] / med / 1e3
-        out.append("| %s | %s | %s | %s | %s | %d | %.2f | `%s` | %d x %d | %d | %.2f | %.0f | %.3f |" % (
-            row["config"], row["kernel"], shape, row["dtype"], lab["what"], lab["bytes"], row[lab["what"]], short(name),
+        same = plain[lab["row"]] if plain and plain[lab["row"]]["shape"] == row["shape"] and plain[lab["row"]]["kernel"] == row["kernel"] \
+            else None
+        out.append("| %s | %s | %s | %s | %s | %d | %s | %.2f | `%s` | %d x %d | %d | %.2f | %.0f | %.3f |" % (
+            row["config"], row["kernel"], shape, row["dtype"], lab["what"], lab["bytes"],
+            "%.2f" % same[lab["what"]] if same else "", row[lab["what"]], short(name),
             grid // wg, wg, len(durs), med, gbs, gbs / HBM_PEAK_GBS))
     return "\n".join(out)
 
@@ -1291,6 +1305,7 @@ def main():
                     help="no GPU: print the `shapes` rows of --bench-json next to the device durations in this "
                          "rocprofv3 --kernel-trace CSV of the same run")
     ap.add_argument("--bench-json", default=None, help="the bench.py output (file) of the profiled run")
+    ap.add_argument("--plain-json", default=None, help="a bench.py output of a run without the profiler, for comparison")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="for rocprofv3 --pmc runs: one 64 MiB device copy (known traffic) then three "
                          "eager steps; prints nothing")
@@ -1303,7 +1318,7 @@ def main():
         print(sweep_summary(args.sweep_summary.split(",")))
         return
     if args.trace_summary:
-        print(trace_summary(args.trace_summary, args.bench_json))
+        print(trace_summary(args.trace_summary, args.bench_json, args.plain_json))
         return
 
     import ctypes

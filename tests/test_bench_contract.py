@@ -83,6 +83,7 @@ def test_trace_summary_cuts_a_kernel_trace_at_the_marker_launches(tmp_path):
     lines = [l for l in text.splitlines() if l.startswith("| cfg2")]
     assert len(lines) == 2
     assert "gn_slice_kernel<__half, 5, true, true>" in lines[0] and "| 256 x 1024 | 4 | 5.20 |" in lines[0]
+    assert "| 10485760 |  | 5.20 |" in lines[0]     # no unprofiled run given: that column stays empty
     assert "gn_slice_kernel<__half, 2, true, false>" in lines[1] and "| 256 x 640 | 3 | 6.00 |" in lines[1]
     assert "| %.0f | %.3f |" % (10485760 / 5.2 / 1e3, 10485760 / 5.2 / 1e3 / 8000.0) in lines[0]
 

@@ -764,6 +764,56 @@ def test_groupnorm_several_writers_per_unit_give_the_bits_of_one(msd, orc, cuda,
     assert msd.status() == 0
 
 
+@pytest.mark.parametrize("cus,xcds", [(256, 1), (64, 2), (128, 4), (512, 16), (228, 6)])
+def test_groupnorm_planned_for_other_chips_runs_right_on_this_one(msd, orc, cuda, cus, xcds):
+    """The launch follows the CU / XCD count the device reports; here other chips are injected
+    through the knobs and the launches they get are run on the real device.  What changes is
+    how many workgroups share a unit and how far apart their block ids are (one XCD count, any
+    power of two; adjacent for one XCD or a count that is not a power of two): the result must
+    not depend on it - equal to the oracle, and to the same launch with one writer bit for bit.
+    Token-major store included (its block layout uses the same stride)."""
+    torch = _torch()
+    lib = msd.load_library()
+    try:
+        assert lib.msd_set_tuning(msd.TUNE_DEVICE_CUS, cus) == 0
+        assert lib.msd_set_tuning(msd.TUNE_DEVICE_XCDS, xcds) == 0
+        for batch, channels, hw, half in ((2, 640, 1024, True), (1, 1280, 256, True), (2, 320, 4096, False),
+                                          (4, 1920, 256, True), (2, 1280, 64, False)):
+            x = orc.normal((batch, channels, hw), seed=cus + xcds + channels, sigma=1.7, mean=0.2)
+            g, b = _affine(orc, channels, cus + channels)
+            code = msd.DTYPE_F16 if half else msd.DTYPE_F32
+            plan = msd.groupnorm_plan(batch, channels, hw, 32, code)
+            if plan[3] > 1:  # several writers: their stride is what the injected XCD count changes
+                assert (batch * 32) % xcds == 0 and xcds & (xcds - 1) == 0 and batch * 32 * plan[3] <= cus
+            xin = orc.round_to_half(x) if half else x
+            xd, gd, bd = _to_dev(xin, cuda, half), _to_dev(g, cuda), _to_dev(b, cuda)
+            got = msd.groupnorm(xd, gd, bd, 32, 1e-5, True)
+            assert lib.msd_set_tuning(msd.TUNE_GN_THREADS, plan[1]) == 0
+            assert lib.msd_set_tuning(msd.TUNE_GN_SPLIT, plan[0]) == 0
+            assert lib.msd_set_tuning(msd.TUNE_GN_WRITERS, 1) == 0
+            one = msd.groupnorm(xd, gd, bd, 32, 1e-5, True)
+            for knob in (msd.TUNE_GN_THREADS, msd.TUNE_GN_SPLIT, msd.TUNE_GN_WRITERS):
+                assert lib.msd_set_tuning(knob, 0) == 0
+            if plan[3] > 1:
+                assert torch.equal(got, one), (cus, xcds, batch, channels, hw, plan)
+            ref = orc.groupnorm(xin, g, b, 32, 1e-5, True)
+            if half:
+                assert_close_f16(got.float().cpu().numpy(), ref, "gn other chip f16")
+            else:
+                assert_close_f32(got.cpu().numpy(), ref, what="gn other chip f32 %s" % ((cus, xcds, batch, channels, hw),))
+            if channels <= 1280:  # token-major store of the same tensor (no SiLU, eps 1e-6)
+                tok = msd.groupnorm_tokens(xd, gd, bd, 32, 1e-6).float().cpu().numpy()
+                ref_t = np.ascontiguousarray(np.transpose(orc.groupnorm(xin, g, b, 32, 1e-6, False), (0, 2, 1)))
+                if half:
+                    assert_close_f16(tok, ref_t, "gn tokens other chip f16")
+                else:
+                    assert_close_f32(tok, ref_t, what="gn tokens other chip f32")
+    finally:
+        for knob in (msd.TUNE_DEVICE_CUS, msd.TUNE_DEVICE_XCDS, msd.TUNE_GN_THREADS, msd.TUNE_GN_SPLIT, msd.TUNE_GN_WRITERS):
+            lib.msd_set_tuning(knob, 0)
+    assert msd.status() == 0
+
+
 def test_groupnorm_many_units_and_register_limits(msd, orc, cuda, gn_writers):
     # more units than scratch slots (never split), and float units that need a split to fit
     for shape, groups, half in [((300, 64, 4, 8), 32, True),     # 9600 units
