@@ -456,3 +456,39 @@ def test_layer_objects_from_cpp_against_golden_files(orc, cuda, tmp_path):
     assert verdicts == ["PASS"] * 7 + ["FAIL", "FAIL"], p.stdout + p.stderr
     assert p.returncode == 2 and out[-1] == "7 of 9 cases passed"
     assert "max diff:" in p.stderr and "Unable to open file" in p.stderr
+
+
+def test_an_earlier_hip_error_of_the_application_is_neither_reported_nor_cleared(msd, cuda):
+    """Launches report the status hipLaunchKernel returns for them.  An error that an unrelated
+    earlier call of the application left in the runtime's per-thread "last error" (here: a
+    hipFree of a pointer nobody allocated) is not mistaken for a failed launch, and it is still
+    there for the application to read afterwards."""
+    import ctypes
+    import torch
+    path = None
+    with open("/proc/self/maps") as f:
+        for line in f:
+            name = line.split()[-1]
+            if "/libamdhip64.so" in name:
+                path = name
+                break
+    assert path, "the HIP runtime is not mapped"
+    hip = ctypes.CDLL(path)
+    hip.hipFree.argtypes = [ctypes.c_void_p]
+    lib = msd.load_library()
+    x = torch.linspace(-4, 4, 4096, device=cuda)
+    y = torch.empty_like(x)
+    want = x * torch.sigmoid(x)
+    torch.cuda.synchronize()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    assert hip.hipGetLastError() == 0
+    try:
+        err = hip.hipFree(ctypes.c_void_p(0x1000))          # the application's own mistake
+        assert err != 0 and hip.hipPeekAtLastError() == err
+        rc = lib.msd_silu(ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(y.data_ptr()), x.numel(), msd.DTYPE_F32, stream)
+        assert rc == 0, "an earlier error of the application came back as the launch's status"
+        assert lib.msd_status(stream) == 0
+        assert hip.hipPeekAtLastError() == err, "the launch cleared the application's last error"
+    finally:
+        hip.hipGetLastError()                               # read it, as the application would; torch checks it too
+    assert torch.allclose(y, want, rtol=1e-5, atol=1e-6)
