@@ -61,7 +61,7 @@ def rule_plan(msd, lib, row):
         lib.msd_set_tuning(msd.TUNE_GN_PLAN_RULE_ONLY, 0)
 
 
-def main(paths):
+def main(paths, out_path=None):
     sys.path.insert(0, REPO)
     msd = importlib.import_module("mobile-stable-diffusion_amd")
     lib = msd.load_library()
@@ -92,9 +92,10 @@ def main(paths):
               "// do not edit by hand).  {bytes per element, output apart from the input, vectors per unit, units,",
               "// slices per unit, lanes, writers per unit}, then the measured time and what the rule alone picks.",
               "// %d rows from %d measured shapes." % (len(out), len(shapes))]
-    with open(os.path.join(HERE, "gn_plan_table.inc"), "w") as f:
+    with open(out_path or os.path.join(HERE, "gn_plan_table.inc"), "w") as f:
         f.write("\n".join(header + out) + "\n")
     print("%d rows from %d shapes" % (len(out), len(shapes)))
+    return out
 
 
 if __name__ == "__main__":

@@ -181,3 +181,86 @@ def test_random_shapes_always_get_a_launch_that_fits(seed):
         lib.msd_set_tuning(msd.TUNE_GN_SPLIT, 0)
         lib.msd_set_tuning(msd.TUNE_GN_THREADS, 0)
         lib.msd_set_tuning(msd.TUNE_GN_WRITERS, 0)
+
+
+def _table_rows():
+    import os
+    import re
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "mobile-stable-diffusion_amd", "csrc",
+                        "gn_plan_table.inc")
+    rows = []
+    for line in open(path):
+        m = re.match(r"\s*\{(\d+),\s*(\d+),\s*(\d+),\s*(\d+),\s*(\d+),\s*(\d+),\s*(\d+)\}", line)
+        if m:
+            rows.append(tuple(int(v) for v in m.groups()))
+    return rows
+
+
+def test_every_row_of_the_table_of_measured_plans_is_the_plan_its_shape_gets():
+    """The table is data written by gn_plan_table.py: each row must name a launch the kernels are
+    built for, and gn_decide must hand exactly that launch to the shape the row is for (on the
+    chip the table belongs to) - and something else, the rule's plan, when the table is off."""
+    rows = _table_rows()
+    assert 20 <= len(rows) <= 200 and len(set(r[:4] for r in rows)) == len(rows)   # one row per shape
+    differs = 0
+    for elt, apart, vectors, units, split, threads, writers in rows:
+        code = msd.DTYPE_F16 if elt == 2 else msd.DTYPE_F32
+        assert units % 32 == 0 and vectors % 10 == 0
+        batch, channels, hw = units // 32, 320, vectors * (16 // elt) // 10      # 10 channels per group
+        got = _check(batch, channels, hw, 32, code, in_place=not apart)
+        assert (got[0], got[1], got[3]) == (split, threads, writers), (elt, apart, vectors, units, got)
+        _knobs(msd, GN_PLAN_RULE_ONLY=1)
+        try:
+            differs += _check(batch, channels, hw, 32, code, in_place=not apart) != got
+        finally:
+            _knobs(msd, GN_PLAN_RULE_ONLY=0)
+    assert differs == len(rows)          # a row exists only where the rule alone picks another plan
+
+
+def test_table_generator_keeps_shipped_plans_within_three_percent_and_writes_rows_only_where_the_rule_differs(tmp_path):
+    """gn_plan_table.py on a synthetic sweep: a shape whose shipped plan is within 3 % of the fastest
+    keeps it, one whose shipped plan is further behind gets the fastest, and no row is written where
+    the rule alone already picks the candidate; away from the tuned batches a rule plan within 1 %
+    of the candidate needs no row either."""
+    import importlib.util
+    import json
+    import os
+    here = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("gn_plan_table", os.path.join(here, "mobile-stable-diffusion_amd", "csrc",
+                                                                               "gn_plan_table.py"))
+    gen = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(gen)
+
+    def text(plan):
+        return "%dx%dx%d" % plan[:3] + (" w%d" % plan[3] if plan[3] > 1 else "")
+
+    def row(batch, c, hw, dtype, in_place, auto, variants):
+        elt = 2 if dtype == "f16" else 4
+        return {"batch": batch, "c": c, "hw": hw, "dtype": dtype, "in_place": in_place, "units": batch * 32,
+                "vectors_per_unit": c // 32 * hw * elt // 16, "auto": text(auto), "variants": {text(p): us for p, us in variants.items()}}
+
+    _knobs(msd, GN_PLAN_RULE_ONLY=1)
+    try:
+        rule_a = msd.groupnorm_plan(2, 320, 4096, 32, msd.DTYPE_F16, in_place=True)     # tuned batch
+        rule_b = msd.groupnorm_plan(2, 640, 4096, 32, msd.DTYPE_F16, in_place=True)
+        rule_c = msd.groupnorm_plan(4, 960, 4096, 32, msd.DTYPE_F16, in_place=True)     # batch 4: not a tuned batch
+    finally:
+        _knobs(msd, GN_PLAN_RULE_ONLY=0)
+    shipped_a, fast_b, fast_c = (4, 768, 2, 1), (8, 640, 2, 1), (4, 960, 4, 1)
+    assert shipped_a != rule_a and fast_b != rule_b and fast_c != rule_c
+    sweep = [
+        row(2, 320, 4096, "f16", True, shipped_a, {shipped_a: 6.10, rule_a: 6.00, (2, 1024, 3, 1): 6.05}),   # within 3 %: stays
+        row(2, 640, 4096, "f16", True, rule_b, {rule_b: 7.50, fast_b: 7.00}),                                # 7 % behind: replaced
+        row(4, 960, 4096, "f16", True, fast_c, {fast_c: 12.00, rule_c: 12.05}),                              # rule within 1 %: no row
+        row(2, 1280, 256, "f16", True, msd.groupnorm_plan(2, 1280, 256, 32, msd.DTYPE_F16, in_place=True),
+            {msd.groupnorm_plan(2, 1280, 256, 32, msd.DTYPE_F16, in_place=True): 3.5}),
+    ]
+    src = tmp_path / "sweep.json"
+    src.write_text(json.dumps({"gn_plan_sweep": sweep}) + "\n")
+    out = tmp_path / "table.inc"
+    rows = gen.main([str(src)], str(out))
+    body = [l for l in out.read_text().splitlines() if l.strip().startswith("{")]
+    assert rows == body and len(body) in (2, 3)
+    assert any("{2, 0,  5120,   64, 4,  768, 1}" in l for l in body)        # the shipped plan kept
+    assert any("{2, 0, 10240,   64, 8,  640, 1}" in l for l in body)        # the faster plan taken
+    assert not any(" 15360,  128," in l for l in body)                      # no row: the rule is as good
