@@ -676,6 +676,69 @@ def test_groupnorm_two_streams_have_private_scratch(msd, orc, cuda):
     assert lib.msd_status(ctypes.c_void_p(s2.cuda_stream)) == 0
 
 
+def test_host_threads_on_streams_of_their_own_get_the_results_of_one_thread(msd, orc, cuda):
+    """Four host threads, each with a stream of its own, call cut and whole GroupNorms (a first call
+    per stream allocates that stream's scratch under the library's lock), LayerNorm and GEGLU at the
+    same time; ctypes drops the interpreter lock for the length of each call.  Every thread must see
+    the bits a single thread gets, and no launch error."""
+    import ctypes
+    import threading
+    torch = _torch()
+    lib = msd.load_library()
+    x = orc.round_to_half(orc.normal((2, 640, 4096), seed=811, sigma=2.0, mean=0.5))      # units cut in slices
+    xs = orc.round_to_half(orc.normal((2, 1280, 256), seed=812, sigma=1.0))               # whole units, several writers
+    rows = orc.round_to_half(orc.normal((2048, 640), seed=813))
+    proj = orc.round_to_half(orc.normal((512, 2 * 1280), seed=814))
+    g, b = _affine(orc, 640, 811)
+    gs, bs = _affine(orc, 1280, 812)
+    gl, bl = _affine(orc, 640, 813)
+    dev = [_to_dev(x, cuda, True), _to_dev(xs, cuda, True), _to_dev(rows, cuda, True), _to_dev(proj, cuda, True)]
+    aff = [_to_dev(v, cuda) for v in (g, b, gs, bs, gl, bl)]
+    torch.cuda.synchronize()
+
+    def work():
+        out = [msd.groupnorm(dev[0], aff[0], aff[1], 32, 1e-5, True),
+               msd.groupnorm(dev[1], aff[2], aff[3], 32, 1e-6, False),
+               msd.layernorm(dev[2], aff[4], aff[5], 1e-5),
+               msd.geglu(dev[3])]
+        inplace = dev[0].clone()
+        msd.groupnorm(inplace, aff[0], aff[1], 32, 1e-5, True, out=inplace)
+        return out + [inplace]
+
+    expect = work()
+    torch.cuda.synchronize()
+    results, errors = {}, []
+
+    def thread(i):
+        try:
+            torch.cuda.set_device(0)
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                got = None
+                for _ in range(10):
+                    got = work()
+                stream.synchronize()
+                results[i] = (got, lib.msd_status(ctypes.c_void_p(stream.cuda_stream)))
+        except Exception as e:  # noqa: BLE001 - reported by the asserting thread
+            errors.append((i, repr(e)))
+
+    threads = [threading.Thread(target=thread, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    torch.cuda.synchronize()
+    assert not errors, errors
+    assert sorted(results) == [0, 1, 2, 3]
+    for i, (got, status) in results.items():
+        assert status == 0, "thread %d" % i
+        for k, (a, e) in enumerate(zip(got, expect)):
+            assert torch.equal(a, e), "thread %d, result %d" % (i, k)
+    assert_close_f16(expect[4].float().cpu().numpy(), orc.groupnorm(x, g, b, 32, 1e-5, True), "threads gn in place")
+    assert_close_f16(expect[0].float().cpu().numpy(), orc.groupnorm(x, g, b, 32, 1e-5, True), "threads gn")
+    assert_close_f16(expect[2].float().cpu().numpy(), orc.layernorm(rows, gl, bl, 1e-5), "threads ln")
+
+
 @pytest.mark.parametrize("batch,channels,hw", [(8, 320, 4096), (4, 640, 4096), (8, 960, 1024), (5, 320, 4096)])
 def test_groupnorm_larger_batches_pick_other_splits(msd, orc, cuda, batch, channels, hw, gn_writers):
     # 128 / 256 units: the launch plan cuts units in two or not at all instead of in four
