@@ -718,7 +718,7 @@ def test_host_threads_on_streams_of_their_own_get_the_results_of_one_thread(msd,
                 for _ in range(10):
                     got = work()
                 stream.synchronize()
-                results[i] = (got, lib.msd_status(ctypes.c_void_p(stream.cuda_stream)))
+                results[i] = (got, lib.msd_status(ctypes.c_void_p(stream.cuda_stream)), msd.gn_fallbacks())
         except Exception as e:  # noqa: BLE001 - reported by the asserting thread
             errors.append((i, repr(e)))
 
@@ -730,12 +730,18 @@ def test_host_threads_on_streams_of_their_own_get_the_results_of_one_thread(msd,
     torch.cuda.synchronize()
     assert not errors, errors
     assert sorted(results) == [0, 1, 2, 3]
-    for i, (got, status) in results.items():
+    ref = orc.groupnorm(x, g, b, 32, 1e-5, True)
+    for i, (got, status, gave_up) in results.items():
         assert status == 0, "thread %d" % i
         for k, (a, e) in enumerate(zip(got, expect)):
-            assert torch.equal(a, e), "thread %d, result %d" % (i, k)
-    assert_close_f16(expect[4].float().cpu().numpy(), orc.groupnorm(x, g, b, 32, 1e-5, True), "threads gn in place")
-    assert_close_f16(expect[0].float().cpu().numpy(), orc.groupnorm(x, g, b, 32, 1e-5, True), "threads gn")
+            if gave_up and k in (0, 4):
+                # a slice that was kept waiting by the other threads' launches computed its sibling's
+                # statistics itself, in another order of summation: right, but not the same bits
+                assert_close_f16(a.float().cpu().numpy(), ref, "thread %d, result %d after %d give-ups" % (i, k, gave_up))
+            else:
+                assert torch.equal(a, e), "thread %d, result %d (msd_gn_fallbacks = %d)" % (i, k, gave_up)
+    assert_close_f16(expect[4].float().cpu().numpy(), ref, "threads gn in place")
+    assert_close_f16(expect[0].float().cpu().numpy(), ref, "threads gn")
     assert_close_f16(expect[2].float().cpu().numpy(), orc.layernorm(rows, gl, bl, 1e-5), "threads ln")
 
 
